@@ -1,0 +1,182 @@
+/*
+ * muon_amd.h -- C ABI of libmuon_amd.so: the MI355X (gfx950) Muon optimizer step.
+ *
+ * The reference (thib-s/Muon) has no FFI of its own: its boundary is the Python module
+ * surface of muon.py.  The entry points below are what a ctypes binding of that module needs
+ * to replace the reference's device work; each one cites the reference lines it replaces.
+ *
+ * Conventions
+ *   - every entry point returns 0 on success and a negative MUON_AMD_E* code on failure;
+ *     muon_amd_last_error() returns a thread-local message for the last failure;
+ *   - nothing here allocates or frees device memory, synchronises the device or the stream,
+ *     or keeps a pointer after returning: tensors, descriptor tables and workspace are owned
+ *     by the caller, and all work is enqueued asynchronously on `stream` (a hipStream_t);
+ *   - pointers named *_dev are device pointers; descriptor tables passed as *_dev must stay
+ *     valid until the enqueued kernels have run;
+ *   - matrices are row-major; "bf16" storage is uint16_t holding the upper half of an fp32.
+ */
+#ifndef MUON_AMD_H
+#define MUON_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MUON_AMD_ABI_VERSION 1
+
+#define MUON_AMD_OK        0
+#define MUON_AMD_EINVAL   (-1)   /* bad argument (null pointer, bad size, misaligned table) */
+#define MUON_AMD_ELAUNCH  (-2)   /* HIP reported an error while enqueuing */
+#define MUON_AMD_EDEVICE  (-3)   /* current device is not gfx950 */
+
+/* Newton-Schulz rounding policy (flags argument of the GEMM / norm entry points). */
+#define MUON_AMD_ROUND_REFERENCE 1  /* round every intermediate to bf16 exactly where the
+                                       reference's bf16 tensor expression does (muon.py:282-287) */
+#define MUON_AMD_ROUND_FUSED     0  /* one bf16 rounding per stored output (closer to fp32) */
+
+/* Source dtype of MuonMatDesc.grad. */
+#define MUON_AMD_SRC_F32   0
+#define MUON_AMD_SRC_BF16  1
+
+/* ------------------------------------------------------------------------------------------
+ * Descriptor of one Muon matrix (the 2-D view rows x cols of a parameter; 4-D conv filters are
+ * viewed as (d0, d1*d2*d3) by the caller, muon.py:11-12).  Arrays of these live in device
+ * memory; the elementwise kernels index them by matrix.
+ *
+ * Workspace roles.  m = min(rows, cols), n = max(rows, cols); *_p are those sizes rounded up to
+ * the GEMM tile of the chunk (zero padded; zero rows/columns stay zero through the iteration).
+ *   direct : rows_p x cols_p  bf16, the matrix in the orientation of the parameter
+ *   transp : cols_p x rows_p  bf16, its transpose
+ * For a wide matrix (rows <= cols) X = direct and X^T = transp; for a tall one the roles swap,
+ * which is how the reference's transpose-if-tall (muon.py:278-279, 289-290) is folded into
+ * indexing instead of a pass of its own.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct MuonMatDesc {
+    void*     grad;        /* rows*cols, fp32 (or bf16 per src_dtype): gradient / NS input    */
+    float*    momentum;    /* rows*cols fp32 momentum buffer, or NULL (plain NS)              */
+    float*    param;       /* rows*cols fp32 parameter, or NULL                               */
+    uint16_t* out;         /* rows*cols bf16 functional output, or NULL                       */
+    uint16_t* u;           /* rows*cols bf16 scratch: update before normalisation             */
+    uint16_t* direct;      /* rows_p x cols_p bf16 normalised matrix, parameter orientation   */
+    uint16_t* transp;      /* cols_p x rows_p bf16 normalised matrix, transposed              */
+    const uint16_t* result;/* rows_p x cols_p bf16: NS output in parameter orientation        */
+    float*    partials;    /* per-block partial sums of squares, indexed by global block id   */
+    float*    denom;       /* one float: (||u||_F + eps) as the reference forms it            */
+    int32_t   rows, cols;
+    int32_t   rows_p, cols_p;
+    int32_t   src_dtype;   /* MUON_AMD_SRC_*                                                  */
+    float     scale;       /* max(1, grad.size(-2)/grad.size(-1))**0.5  (muon.py:14)          */
+    int32_t   part_begin;  /* first global block id of this matrix in the momentum launch     */
+    int32_t   part_end;    /* one past the last                                               */
+} MuonMatDesc;
+
+/* One NT GEMM  acc[i][j] = sum_k P[i][k] * Q[j][k]  over a padded matrix, with the epilogue
+ *     t1 = alpha*acc ; t2 = beta*D[i][j] ; (both rounded to bf16 under ROUND_REFERENCE)
+ *     o  = bf16(t1 + t2)          -> C[i][j]  and  CT[j][i]
+ *     o2 = bf16(gamma * o)        -> C2[i][j] and  C2T[j][i]
+ * Any of D, C, CT, C2, C2T may be NULL.  When CT == C the job list only covers tiles with
+ * j0 >= i0 and the kernel mirrors them (it skips the mirror store on diagonal tiles).
+ * Replaces the functional roles of the reference's three Triton kernels:
+ *   ns_line_1 (A = X X^T, muon.py:349-456), ns_line_2 (alpha A A^T + beta A, muon.py:464-588),
+ *   ns_line_3 (a X + B X, muon.py:639-746).                                                   */
+typedef struct MuonGemmDesc {
+    const uint16_t* P;  const uint16_t* Q;  const uint16_t* D;
+    uint16_t* C;  uint16_t* CT;  uint16_t* C2;  uint16_t* C2T;
+    int32_t ldp, ldq, ldd, ldc, ldct;   /* leading dimensions in elements, multiples of 8     */
+    int32_t K;                          /* multiple of 64                                     */
+    int32_t rows, colsn;                /* padded extent of the output (multiples of the tile) */
+} MuonGemmDesc;
+
+/* One output tile of one matrix. */
+typedef struct MuonTileJob {
+    int32_t desc;   /* index into the MuonGemmDesc table of the launch */
+    int32_t i0;     /* first output row  (multiple of the tile)        */
+    int32_t j0;     /* first output col  (multiple of the tile)        */
+    int32_t diag;   /* 1 when i0 == j0 of a mirrored (symmetric) GEMM  */
+} MuonTileJob;
+
+/* One tensor of the auxiliary Adam group. */
+typedef struct MuonAdamDesc {
+    float* param;        /* numel fp32, or NULL when `update` is used instead                 */
+    const float* grad;   /* numel fp32                                                        */
+    float* exp_avg;      /* numel fp32                                                        */
+    float* exp_avg_sq;   /* numel fp32                                                        */
+    float* update;       /* numel fp32 functional output (adam_update's return), or NULL      */
+    int64_t numel;
+} MuonAdamDesc;
+
+int         muon_amd_abi_version(void);
+const char* muon_amd_last_error(void);
+
+/* sizeof() of the structs above, so that a binding can check its own layout. */
+size_t muon_amd_sizeof_mat_desc(void);
+size_t muon_amd_sizeof_gemm_desc(void);
+size_t muon_amd_sizeof_tile_job(void);
+size_t muon_amd_sizeof_adam_desc(void);
+
+/* Elements each block of the flat elementwise launches covers (momentum, apply, adam), and
+ * the edge of the square tile of the normalise/transposing launch. */
+int muon_amd_elementwise_block_elems(void);
+int muon_amd_normalize_tile(void);
+
+/* GEMM tile classes.  tile_class 0: 128x128 output tile, 256 threads; 1: 256x256, 512 threads.
+ * Returns the tile edge, or a negative code for an unknown class. */
+int muon_amd_gemm_tile(int tile_class);
+
+/* ---- host-side validation (no GPU work): checks host copies of the tables a launch will
+ *      use against what the kernels assume.  Call before uploading them.                 ---- */
+int muon_amd_validate_gemm(const MuonGemmDesc* descs_host, int ndesc,
+                           const MuonTileJob* jobs_host, int njobs, int tile_class);
+int muon_amd_validate_mats(const MuonMatDesc* descs_host, int nmat,
+                           const int32_t* block_prefix_host, const int32_t* tile_prefix_host,
+                           int tile_edge);
+
+/* ---- Muon elementwise stages ------------------------------------------------------------ */
+
+/* Momentum EMA + Nesterov blend + bf16 cast + per-block sum of squares
+ * (muon.py:9-10 and the cast of muon.py:277).  block_prefix_dev[nmat+1] maps block -> matrix.
+ *   momentum <- lerp(momentum, grad, one_minus_beta);
+ *   u = nesterov ? lerp(grad, momentum, beta) : momentum       (lerp = torch's two-branch rule)
+ * With mutate_grad != 0 and nesterov, u is also written back into grad as the reference does.
+ * A matrix whose descriptor has momentum == NULL is only cast (u = grad).                    */
+int muon_amd_momentum(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
+                      int nblocks, float one_minus_beta, float beta, int nesterov,
+                      int mutate_grad, void* stream);
+
+/* denom = ||u||_F + eps per matrix from the partial sums (muon.py:282).  Under
+ * MUON_AMD_ROUND_REFERENCE the norm and the sum are rounded to bf16 as the reference's bf16
+ * tensors are. */
+int muon_amd_norm_finalize(const MuonMatDesc* descs_dev, int nmat, float eps, int flags,
+                           void* stream);
+
+/* direct = bf16(u / denom) (zero padded), transp = direct^T (muon.py:278-282).
+ * tile_prefix_dev[nmat+1] maps block -> matrix over (rows_p/T)*(cols_p/T) tiles. */
+int muon_amd_normalize(const MuonMatDesc* descs_dev, const int32_t* tile_prefix_dev, int nmat,
+                       int ntiles, void* stream);
+
+/* One grouped GEMM launch over a tile job list (see MuonGemmDesc). */
+int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
+                     int tile_class, float alpha, float beta, float gamma, int flags,
+                     void* stream);
+
+/* result -> update = bf16(result * scale) (muon.py:14);  if param: param <- param*wd_factor
+ * - lr*update (muon.py:98-99); if out: out <- update (what muon_update returns, muon.py:15). */
+int muon_amd_apply(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
+                   int nblocks, float lr, float wd_factor, void* stream);
+
+/* ---- auxiliary Adam (muon.py:104-109 and 255-258) ---------------------------------------- */
+/* m <- lerp(m, g, w1); v <- lerp(v, g*g, w2)  with w1 = 1-beta1, w2 = 1-beta2;
+ * upd = (m/bias1) / (sqrt(v/bias2) + eps);  param <- param*wd_factor - lr*upd  (or update<-upd)
+ * w1, w2, bias1 = 1-beta1**step and bias2 = 1-beta2**step are computed by the caller in double
+ * (as the reference's Python does) and passed rounded to float. */
+int muon_amd_adam(const MuonAdamDesc* descs_dev, const int32_t* block_prefix_dev, int ntensors,
+                  int nblocks, float lr, float wd_factor, float w1, float w2, float eps,
+                  float bias1, float bias2, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MUON_AMD_H */

@@ -1,0 +1,451 @@
+// HBM-bound stages of the Muon step for gfx950: momentum/Nesterov/cast, Frobenius norm,
+// normalise+transpose, parameter apply, and the auxiliary Adam update.
+//
+// All launches are "grouped": one launch covers every matrix (tensor) of a chunk.  A block
+// finds its matrix by a binary search in a small prefix table and then streams a fixed-size
+// contiguous range of it with 16-byte accesses, so a step costs a handful of launches however
+// many parameters the model has.
+#include "common.h"
+
+namespace muon_amd {
+
+constexpr int EW_THREADS = 256;
+constexpr int EW_VEC = 4;                                       // fp32 elements per access
+constexpr int EW_ITERS = 8;
+constexpr int EW_BLOCK_ELEMS = EW_THREADS * EW_VEC * EW_ITERS;  // 8192 elements per block
+constexpr int NT_TILE = 64;                                     // normalise/transposing tile edge
+
+__device__ __forceinline__ bool aligned_to(const void* p, uintptr_t a) {
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+// Sum of `v` over a 256-thread block, valid in thread 0.
+__device__ __forceinline__ float block_sum_256(float v, float* smem4) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) smem4[wave] = v;
+    __syncthreads();
+    return (smem4[0] + smem4[1]) + (smem4[2] + smem4[3]);
+}
+
+// ------------------------------------------------------------------------------------------
+// momentum: muon.py:9-10 + the bf16 cast of muon.py:277 + partial sums for muon.py:282
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float momentum_one(float g, float* m_io, bool has_m, float w,
+                                              float beta, int nesterov, float* g_out) {
+    if (!has_m) return g;
+    const float m_new = lerp_torch(*m_io, g, w);          // momentum.lerp_(grad, 1 - beta)
+    *m_io = m_new;
+    if (!nesterov) return m_new;
+    const float u = lerp_torch(g, m_new, beta);           // grad.lerp_(momentum, beta)
+    *g_out = u;
+    return u;
+}
+
+__global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
+    const MuonMatDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, float w,
+    float beta, int nesterov, int mutate_grad) {
+    __shared__ float red[4];
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonMatDesc d = descs[mi];
+    const int64_t numel = static_cast<int64_t>(d.rows) * d.cols;
+    const int64_t base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
+    const bool has_m = d.momentum != nullptr;
+    const bool write_g = has_m && nesterov && mutate_grad;
+    const bool src_bf16 = d.src_dtype == MUON_AMD_SRC_BF16;
+    float* __restrict__ mom = d.momentum;
+    uint16_t* __restrict__ u = d.u;
+    float ss = 0.f;
+
+    const bool vec_ok = !src_bf16 && aligned_to(d.grad, 16) && aligned_to(mom, 16) &&
+                        aligned_to(u, 8) && (base + EW_BLOCK_ELEMS <= numel);
+    if (vec_ok) {
+        float* __restrict__ g = static_cast<float*>(d.grad);
+        float4 gv[EW_ITERS], mv[EW_ITERS];
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            gv[it] = *reinterpret_cast<const float4*>(g + e);
+            mv[it] = has_m ? *reinterpret_cast<const float4*>(mom + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            float gg[4] = {gv[it].x, gv[it].y, gv[it].z, gv[it].w};
+            float mm[4] = {mv[it].x, mv[it].y, mv[it].z, mv[it].w};
+            float uu[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float gout = gg[k];
+                uu[k] = momentum_one(gg[k], &mm[k], has_m, w, beta, nesterov, &gout);
+                gg[k] = gout;
+                const float ub = round_bf(uu[k]);
+                ss = fmaf(ub, ub, ss);
+            }
+            if (has_m) *reinterpret_cast<float4*>(mom + e) = make_float4(mm[0], mm[1], mm[2], mm[3]);
+            if (write_g) *reinterpret_cast<float4*>(g + e) = make_float4(gg[0], gg[1], gg[2], gg[3]);
+            uint2 pk;
+            pk.x = pack2bf(uu[0], uu[1]);
+            pk.y = pack2bf(uu[2], uu[3]);
+            *reinterpret_cast<uint2*>(u + e) = pk;
+        }
+    } else {
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+#pragma unroll
+            for (int k = 0; k < EW_VEC; ++k) {
+                const int64_t e = e0 + k;
+                if (e >= numel) break;
+                float gval = src_bf16 ? bf2f(static_cast<const uint16_t*>(d.grad)[e])
+                                      : static_cast<const float*>(d.grad)[e];
+                float mval = has_m ? mom[e] : 0.f;
+                float gout = gval;
+                const float uval = momentum_one(gval, &mval, has_m, w, beta, nesterov, &gout);
+                if (has_m) mom[e] = mval;
+                if (write_g) static_cast<float*>(d.grad)[e] = gout;
+                const uint16_t ub = f2bf(uval);
+                u[e] = ub;
+                const float uf = bf2f(ub);
+                ss = fmaf(uf, uf, ss);
+            }
+        }
+    }
+    const float total = block_sum_256(ss, red);
+    if (threadIdx.x == 0) d.partials[b] = total;
+}
+
+// ------------------------------------------------------------------------------------------
+// norm finalize: muon.py:282  (X.norm(dim=(-2,-1)) + 1e-7)
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void norm_finalize_kernel(const MuonMatDesc* __restrict__ descs,
+                                                            float eps, int round_reference) {
+    const MuonMatDesc d = descs[blockIdx.x];
+    float s = 0.f;
+    for (int i = d.part_begin + threadIdx.x; i < d.part_end; i += 64) s += d.partials[i];
+    s = wave_sum(s);
+    if (threadIdx.x == 0) {
+        float nrm = sqrtf(s);
+        float den;
+        if (round_reference) {
+            nrm = round_bf(nrm);           // the norm of a bf16 tensor is a bf16 tensor
+            den = round_bf(nrm + eps);     // bf16 tensor + python scalar -> bf16 tensor
+        } else {
+            den = nrm + eps;
+        }
+        *d.denom = den;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// normalise + transpose + zero pad:  direct = bf16(u / denom), transp = direct^T
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __restrict__ descs,
+                                                         const int32_t* __restrict__ prefix,
+                                                         int nmat) {
+    __shared__ uint16_t tile[NT_TILE][NT_TILE + 2];
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonMatDesc d = descs[mi];
+    const int lb = b - prefix[mi];
+    const int tiles_c = d.cols_p / NT_TILE;
+    const int R0 = (lb / tiles_c) * NT_TILE, C0 = (lb % tiles_c) * NT_TILE;
+    const float den = *d.denom;
+    const uint16_t* __restrict__ u = d.u;
+    const bool vec_ok = (d.cols % 8 == 0) && aligned_to(u, 16);
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int q = threadIdx.x + i * 256;
+        const int r = q >> 3, cc = (q & 7) * 8;
+        const int gr = R0 + r, gc = C0 + cc;
+        uint16_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = 0;
+        if (gr < d.rows) {
+            const int64_t off = static_cast<int64_t>(gr) * d.cols + gc;
+            if (vec_ok && gc + 8 <= d.cols) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(u + off);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v[2 * k] = static_cast<uint16_t>(w[k] & 0xffffu);
+                    v[2 * k + 1] = static_cast<uint16_t>(w[k] >> 16);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (gc + k < d.cols) v[k] = u[off + k];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (gc + k < d.cols) v[k] = f2bf(bf2f(v[k]) / den);
+        }
+        uint4 o;
+        o.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
+        o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
+        o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
+        o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
+        *reinterpret_cast<uint4*>(d.direct + static_cast<int64_t>(gr) * d.cols_p + gc) = o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) tile[r][cc + k] = v[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int q = threadIdx.x + i * 256;
+        const int tr = q >> 3, tc = (q & 7) * 8;   // transposed tile: row tr (a source column)
+        uint16_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = tile[tc + k][tr];
+        uint4 o;
+        o.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
+        o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
+        o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
+        o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
+        *reinterpret_cast<uint4*>(d.transp + static_cast<int64_t>(C0 + tr) * d.rows_p + R0 + tc) = o;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// apply: muon.py:14 (aspect scale, in bf16), muon.py:98-99 (decoupled decay + step)
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __restrict__ descs,
+                                                            const int32_t* __restrict__ prefix,
+                                                            int nmat, float neg_lr, float wd_factor) {
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonMatDesc d = descs[mi];
+    const int64_t numel = static_cast<int64_t>(d.rows) * d.cols;
+    const int64_t base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
+    float* __restrict__ p = d.param;
+    uint16_t* __restrict__ out = d.out;
+    const uint16_t* __restrict__ res = d.result;
+    const float scale = d.scale;
+    const bool vec_ok = (d.cols % 4 == 0) && aligned_to(p, 16) && aligned_to(out, 8) &&
+                        (base + EW_BLOCK_ELEMS <= numel);
+    if (vec_ok) {
+        float4 pv[EW_ITERS];
+        uint2 ov[EW_ITERS];
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
+            ov[it] = *reinterpret_cast<const uint2*>(res + static_cast<int64_t>(rr) * d.cols_p + cc);
+            pv[it] = p ? *reinterpret_cast<const float4*>(p + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            uint16_t o[4] = {static_cast<uint16_t>(ov[it].x & 0xffffu), static_cast<uint16_t>(ov[it].x >> 16),
+                             static_cast<uint16_t>(ov[it].y & 0xffffu), static_cast<uint16_t>(ov[it].y >> 16)};
+            float pp[4] = {pv[it].x, pv[it].y, pv[it].z, pv[it].w};
+            float us[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                us[k] = round_bf(bf2f(o[k]) * scale);
+                pp[k] = fmaf(neg_lr, us[k], pp[k] * wd_factor);
+            }
+            if (p) *reinterpret_cast<float4*>(p + e) = make_float4(pp[0], pp[1], pp[2], pp[3]);
+            if (out) {
+                uint2 pk;
+                pk.x = pack2bf(us[0], us[1]);
+                pk.y = pack2bf(us[2], us[3]);
+                *reinterpret_cast<uint2*>(out + e) = pk;
+            }
+        }
+    } else {
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+#pragma unroll
+            for (int k = 0; k < EW_VEC; ++k) {
+                const int64_t e = e0 + k;
+                if (e >= numel) break;
+                const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
+                const float us = round_bf(bf2f(res[static_cast<int64_t>(rr) * d.cols_p + cc]) * scale);
+                if (p) p[e] = fmaf(neg_lr, us, p[e] * wd_factor);
+                if (out) out[e] = f2bf(us);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// auxiliary Adam: muon.py:104-109 + 257-258
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float adam_one(float g, float* m, float* v, float w1, float w2,
+                                          float eps, float bias1, float bias2) {
+    *m = lerp_torch(*m, g, w1);
+    *v = lerp_torch(*v, g * g, w2);
+    const float mc = *m / bias1;
+    const float vc = *v / bias2;
+    return mc / (sqrtf(vc) + eps);
+}
+
+__global__ __launch_bounds__(EW_THREADS) void adam_kernel(const MuonAdamDesc* __restrict__ descs,
+                                                           const int32_t* __restrict__ prefix,
+                                                           int ntensors, float neg_lr,
+                                                           float wd_factor, float w1, float w2,
+                                                           float eps, float bias1, float bias2) {
+    const int b = blockIdx.x;
+    const int ti = find_segment(prefix, ntensors, b);
+    const MuonAdamDesc d = descs[ti];
+    const int64_t numel = d.numel;
+    const int64_t base = static_cast<int64_t>(b - prefix[ti]) * EW_BLOCK_ELEMS;
+    float* __restrict__ p = d.param;
+    const float* __restrict__ g = d.grad;
+    float* __restrict__ m = d.exp_avg;
+    float* __restrict__ v = d.exp_avg_sq;
+    float* __restrict__ upd = d.update;
+    const bool vec_ok = aligned_to(p, 16) && aligned_to(g, 16) && aligned_to(m, 16) &&
+                        aligned_to(v, 16) && aligned_to(upd, 16) &&
+                        (base + EW_BLOCK_ELEMS <= numel);
+    if (vec_ok) {
+        float4 gv[EW_ITERS], mv[EW_ITERS], vv[EW_ITERS], pv[EW_ITERS];
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            gv[it] = *reinterpret_cast<const float4*>(g + e);
+            mv[it] = *reinterpret_cast<const float4*>(m + e);
+            vv[it] = *reinterpret_cast<const float4*>(v + e);
+            pv[it] = p ? *reinterpret_cast<const float4*>(p + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+            float gg[4] = {gv[it].x, gv[it].y, gv[it].z, gv[it].w};
+            float mm[4] = {mv[it].x, mv[it].y, mv[it].z, mv[it].w};
+            float v2[4] = {vv[it].x, vv[it].y, vv[it].z, vv[it].w};
+            float pp[4] = {pv[it].x, pv[it].y, pv[it].z, pv[it].w};
+            float uu[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uu[k] = adam_one(gg[k], &mm[k], &v2[k], w1, w2, eps, bias1, bias2);
+                pp[k] = fmaf(neg_lr, uu[k], pp[k] * wd_factor);
+            }
+            *reinterpret_cast<float4*>(m + e) = make_float4(mm[0], mm[1], mm[2], mm[3]);
+            *reinterpret_cast<float4*>(v + e) = make_float4(v2[0], v2[1], v2[2], v2[3]);
+            if (p) *reinterpret_cast<float4*>(p + e) = make_float4(pp[0], pp[1], pp[2], pp[3]);
+            if (upd) *reinterpret_cast<float4*>(upd + e) = make_float4(uu[0], uu[1], uu[2], uu[3]);
+        }
+    } else {
+        for (int it = 0; it < EW_ITERS; ++it) {
+            const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+#pragma unroll
+            for (int k = 0; k < EW_VEC; ++k) {
+                const int64_t e = e0 + k;
+                if (e >= numel) break;
+                float mm = m[e], v2 = v[e];
+                const float uu = adam_one(g[e], &mm, &v2, w1, w2, eps, bias1, bias2);
+                m[e] = mm;
+                v[e] = v2;
+                if (p) p[e] = fmaf(neg_lr, uu, p[e] * wd_factor);
+                if (upd) upd[e] = uu;
+            }
+        }
+    }
+}
+
+}  // namespace muon_amd
+
+using namespace muon_amd;
+
+extern "C" {
+
+int muon_amd_elementwise_block_elems(void) { return EW_BLOCK_ELEMS; }
+int muon_amd_normalize_tile(void) { return NT_TILE; }
+
+int muon_amd_validate_mats(const MuonMatDesc* descs, int nmat, const int32_t* block_prefix,
+                           const int32_t* tile_prefix, int tile_edge) {
+    MUON_REQUIRE(descs && block_prefix && tile_prefix, "validate_mats: null table");
+    MUON_REQUIRE(nmat > 0, "validate_mats: nmat=%d", nmat);
+    MUON_REQUIRE(tile_edge > 0 && tile_edge % NT_TILE == 0, "validate_mats: tile_edge=%d", tile_edge);
+    MUON_REQUIRE(block_prefix[0] == 0 && tile_prefix[0] == 0, "validate_mats: prefix must start at 0");
+    for (int i = 0; i < nmat; ++i) {
+        const MuonMatDesc& d = descs[i];
+        MUON_REQUIRE(d.rows > 0 && d.cols > 0, "mat %d: rows=%d cols=%d", i, d.rows, d.cols);
+        MUON_REQUIRE(d.rows_p >= d.rows && d.cols_p >= d.cols && d.rows_p % tile_edge == 0 &&
+                         d.cols_p % tile_edge == 0,
+                     "mat %d: padded %dx%d does not cover %dx%d in tiles of %d", i, d.rows_p,
+                     d.cols_p, d.rows, d.cols, tile_edge);
+        MUON_REQUIRE(d.grad && d.u && d.direct && d.transp && d.result && d.partials && d.denom,
+                     "mat %d: null workspace or source pointer", i);
+        MUON_REQUIRE(d.param || d.out, "mat %d: neither param nor out given", i);
+        MUON_REQUIRE(d.src_dtype == MUON_AMD_SRC_F32 || d.src_dtype == MUON_AMD_SRC_BF16,
+                     "mat %d: src_dtype=%d", i, d.src_dtype);
+        MUON_REQUIRE(d.src_dtype == MUON_AMD_SRC_F32 || d.momentum == nullptr,
+                     "mat %d: momentum needs an fp32 gradient", i);
+        MUON_REQUIRE((reinterpret_cast<uintptr_t>(d.direct) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(d.transp) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(d.result) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(d.u) % 16) == 0,
+                     "mat %d: workspace pointers must be 16-byte aligned", i);
+        const int64_t numel = static_cast<int64_t>(d.rows) * d.cols;
+        const int64_t nblk = (numel + EW_BLOCK_ELEMS - 1) / EW_BLOCK_ELEMS;
+        MUON_REQUIRE(block_prefix[i + 1] - block_prefix[i] == nblk,
+                     "mat %d: block prefix gives %d blocks, need %lld", i,
+                     block_prefix[i + 1] - block_prefix[i], static_cast<long long>(nblk));
+        MUON_REQUIRE(d.part_end - d.part_begin == nblk, "mat %d: partial range %d..%d, need %lld blocks",
+                     i, d.part_begin, d.part_end, static_cast<long long>(nblk));
+        MUON_REQUIRE(d.part_begin == block_prefix[i], "mat %d: part_begin %d != block prefix %d", i,
+                     d.part_begin, block_prefix[i]);
+        const int64_t ntile = static_cast<int64_t>(d.rows_p / NT_TILE) * (d.cols_p / NT_TILE);
+        MUON_REQUIRE(tile_prefix[i + 1] - tile_prefix[i] == ntile, "mat %d: tile prefix gives %d tiles, need %lld",
+                     i, tile_prefix[i + 1] - tile_prefix[i], static_cast<long long>(ntile));
+    }
+    return MUON_AMD_OK;
+}
+
+int muon_amd_momentum(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
+                      int nblocks, float one_minus_beta, float beta, int nesterov,
+                      int mutate_grad, void* stream) {
+    MUON_REQUIRE(descs_dev && block_prefix_dev, "momentum: null table");
+    MUON_REQUIRE(nmat > 0 && nblocks > 0, "momentum: nmat=%d nblocks=%d", nmat, nblocks);
+    hipLaunchKernelGGL(momentum_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, nmat,
+                       one_minus_beta, beta, nesterov, mutate_grad);
+    return check_launch("momentum");
+}
+
+int muon_amd_norm_finalize(const MuonMatDesc* descs_dev, int nmat, float eps, int flags,
+                           void* stream) {
+    MUON_REQUIRE(descs_dev, "norm_finalize: null table");
+    MUON_REQUIRE(nmat > 0, "norm_finalize: nmat=%d", nmat);
+    hipLaunchKernelGGL(norm_finalize_kernel, dim3(nmat), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, eps,
+                       (flags & MUON_AMD_ROUND_REFERENCE) ? 1 : 0);
+    return check_launch("norm_finalize");
+}
+
+int muon_amd_normalize(const MuonMatDesc* descs_dev, const int32_t* tile_prefix_dev, int nmat,
+                       int ntiles, void* stream) {
+    MUON_REQUIRE(descs_dev && tile_prefix_dev, "normalize: null table");
+    MUON_REQUIRE(nmat > 0 && ntiles > 0, "normalize: nmat=%d ntiles=%d", nmat, ntiles);
+    hipLaunchKernelGGL(normalize_kernel, dim3(ntiles), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, tile_prefix_dev, nmat);
+    return check_launch("normalize");
+}
+
+int muon_amd_apply(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
+                   int nblocks, float lr, float wd_factor, void* stream) {
+    MUON_REQUIRE(descs_dev && block_prefix_dev, "apply: null table");
+    MUON_REQUIRE(nmat > 0 && nblocks > 0, "apply: nmat=%d nblocks=%d", nmat, nblocks);
+    hipLaunchKernelGGL(apply_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, nmat, -lr,
+                       wd_factor);
+    return check_launch("apply");
+}
+
+int muon_amd_adam(const MuonAdamDesc* descs_dev, const int32_t* block_prefix_dev, int ntensors,
+                  int nblocks, float lr, float wd_factor, float w1, float w2, float eps,
+                  float bias1, float bias2, void* stream) {
+    MUON_REQUIRE(descs_dev && block_prefix_dev, "adam: null table");
+    MUON_REQUIRE(ntensors > 0 && nblocks > 0, "adam: ntensors=%d nblocks=%d", ntensors, nblocks);
+    MUON_REQUIRE(bias1 != 0.f && bias2 != 0.f, "adam: zero bias correction");
+    hipLaunchKernelGGL(adam_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, ntensors,
+                       -lr, wd_factor, w1, w2, eps, bias1, bias2);
+    return check_launch("adam");
+}
+
+}  // extern "C"

@@ -1,0 +1,170 @@
+"""Device-side driver of the grouped Muon / Adam launches (torch for memory and streams only)."""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+import torch
+
+from . import _lib, plan as _plan
+
+DEFAULT_WORKSPACE_CAP = int(os.environ.get("MUON_AMD_WORKSPACE_BYTES", 16 << 30))
+
+
+def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise _lib.MuonAmdError(
+            f"{what} is on {t.device}: muon_amd runs on an MI355X (gfx950) GPU only and has no "
+            "CPU implementation")
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _upload(arr: np.ndarray, device) -> torch.Tensor:
+    """Async host->device copy of a table through pinned staging (no stream or host sync)."""
+    host = torch.from_numpy(arr.view(np.uint8).reshape(-1)).pin_memory()
+    return host.to(device, non_blocking=True)
+
+
+class _ChunkRuntime:
+    def __init__(self, chunk: _plan.ChunkPlan, base: int, device):
+        lib = _lib.load()
+        self.chunk = chunk
+        self.device = device
+        gemm = chunk.gemm_descs(base)
+        for ph in range(5):
+            jobs = chunk.sym_jobs if ph in (_plan.PH_SYRK, _plan.PH_POLY) else chunk.full_jobs
+            _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(gemm[ph]), chunk.nmat,
+                                                  _lib.host_ptr(jobs), len(jobs), chunk.tile_class),
+                       "validate_gemm")
+        self.mat_template = chunk.mat_descs(base)
+        # one static device blob: gemm descs | sym jobs | full jobs | block prefix | tile prefix
+        parts = [gemm.reshape(-1).view(np.uint8), chunk.sym_jobs.view(np.uint8),
+                 chunk.full_jobs.view(np.uint8), chunk.block_prefix.view(np.uint8),
+                 chunk.tile_prefix.view(np.uint8)]
+        offs, blob, cur = [], [], 0
+        for p in parts:
+            offs.append(cur)
+            pad = (-len(p)) % 256
+            blob.append(p)
+            if pad:
+                blob.append(np.zeros(pad, dtype=np.uint8))
+            cur += len(p) + pad
+        self.static = _upload(np.concatenate(blob), device)
+        b = self.static.data_ptr()
+        self.gemm_ptr = [b + offs[0] + ph * chunk.nmat * _lib.GEMM_DESC.itemsize for ph in range(5)]
+        self.sym_jobs_ptr = b + offs[1]
+        self.full_jobs_ptr = b + offs[2]
+        self.block_prefix_ptr = b + offs[3]
+        self.tile_prefix_ptr = b + offs[4]
+        self.mat_dev = None
+        self.mat_key = None
+
+    def bind(self, grads, momenta, params, outs, scales, src_dtypes):
+        """(Re)upload the matrix descriptors if any tensor address changed since the last call."""
+        key = (tuple(grads), tuple(momenta), tuple(params), tuple(outs), tuple(scales), tuple(src_dtypes))
+        if key == self.mat_key:
+            return
+        lib = _lib.load()
+        d = self.mat_template.copy()
+        d["grad"] = grads
+        d["momentum"] = momenta
+        d["param"] = params
+        d["out"] = outs
+        d["scale"] = scales
+        d["src_dtype"] = src_dtypes
+        _lib.check(lib.muon_amd_validate_mats(_lib.host_ptr(d), self.chunk.nmat,
+                                              _lib.host_ptr(self.chunk.block_prefix),
+                                              _lib.host_ptr(self.chunk.tile_prefix), self.chunk.tile),
+                   "validate_mats")
+        self.mat_dev = _upload(d, self.device)
+        self.mat_key = key
+
+    def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor):
+        lib = _lib.load()
+        c = self.chunk
+        s = _stream_ptr(self.device)
+        flags = _lib.ROUND_REFERENCE if c.reference_rounding else _lib.ROUND_FUSED
+        mats = self.mat_dev.data_ptr()
+        _lib.check(lib.muon_amd_momentum(mats, self.block_prefix_ptr, c.nmat, c.nblocks,
+                                         one_minus_beta, beta, int(nesterov), int(mutate_grad), s), "momentum")
+        _lib.check(lib.muon_amd_norm_finalize(mats, c.nmat, eps, flags, s), "norm_finalize")
+        _lib.check(lib.muon_amd_normalize(mats, self.tile_prefix_ptr, c.nmat, c.ntiles, s), "normalize")
+        for it in range(c.steps):
+            for ph in (_plan.PH_SYRK, _plan.PH_POLY):
+                al, be, ga = c.phase_scalars(ph)
+                _lib.check(lib.muon_amd_ns_gemm(self.gemm_ptr[ph], self.sym_jobs_ptr, len(c.sym_jobs),
+                                                c.tile_class, al, be, ga, flags, s), "ns_gemm")
+            ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
+            al, be, ga = c.phase_scalars(ph)
+            _lib.check(lib.muon_amd_ns_gemm(self.gemm_ptr[ph], self.full_jobs_ptr, len(c.full_jobs),
+                                            c.tile_class, al, be, ga, flags, s), "ns_gemm")
+        _lib.check(lib.muon_amd_apply(mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply")
+
+
+class MuonGroupEngine:
+    """Runs the Muon update of a fixed list of matrix shapes on one device.
+
+    Built once per (shapes, steps, rounding); each `run` takes the current tensor addresses.
+    """
+
+    def __init__(self, shapes, device, steps: int = 5, reference_rounding: bool = True,
+                 workspace_cap: int | None = None):
+        _lib.load()
+        self.device = torch.device(device)
+        self.shapes = [(int(r), int(c)) for r, c in shapes]
+        cap = DEFAULT_WORKSPACE_CAP if workspace_cap is None else int(workspace_cap)
+        self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap)
+        ws_bytes = max(c.workspace_bytes for c in self.chunks)
+        self.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self.device)
+        base = self.workspace.data_ptr()
+        assert base % 256 == 0
+        self.runtimes = [_ChunkRuntime(c, base, self.device) for c in self.chunks]
+
+    def run(self, grads, momenta, params, outs, scales, src_dtypes, *, beta, nesterov, mutate_grad,
+            eps, lr, weight_decay):
+        """All arguments are per-matrix lists in the order of `shapes` (device addresses or 0)."""
+        one_minus_beta = 1 - beta                      # python double, as muon.py:9
+        wd_factor = 1 - lr * weight_decay              # python double, as muon.py:98
+        for rt in self.runtimes:
+            idx = [lay.index for lay in rt.chunk.layouts]
+            rt.bind([grads[i] for i in idx], [momenta[i] for i in idx], [params[i] for i in idx],
+                    [outs[i] for i in idx], [scales[i] for i in idx], [src_dtypes[i] for i in idx])
+            rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor)
+
+
+class AdamGroupEngine:
+    """Fused auxiliary-Adam launch over a fixed list of tensors."""
+
+    def __init__(self, numels, device):
+        _lib.load()
+        self.device = torch.device(device)
+        self.numels = [int(n) for n in numels]
+        self.prefix = _plan.adam_block_prefix(self.numels)
+        self.nblocks = int(self.prefix[-1])
+        self.prefix_dev = _upload(self.prefix, self.device)
+        self.desc_dev = None
+        self.key = None
+
+    def run(self, params, grads, exp_avgs, exp_avg_sqs, updates, *, lr, weight_decay, betas, eps, step):
+        key = (tuple(params), tuple(grads), tuple(exp_avgs), tuple(exp_avg_sqs), tuple(updates))
+        if key != self.key:
+            d = np.zeros(len(self.numels), dtype=_lib.ADAM_DESC)
+            d["param"] = params
+            d["grad"] = grads
+            d["exp_avg"] = exp_avgs
+            d["exp_avg_sq"] = exp_avg_sqs
+            d["update"] = updates
+            d["numel"] = self.numels
+            self.desc_dev = _upload(d, self.device)
+            self.key = key
+        lib = _lib.load()
+        w1 = 1 - betas[0]                              # python doubles, as muon.py:105-108
+        w2 = 1 - betas[1]
+        bias1 = 1 - betas[0] ** step
+        bias2 = 1 - betas[1] ** step
+        _lib.check(lib.muon_amd_adam(self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels),
+                                     self.nblocks, lr, 1 - lr * weight_decay, w1, w2, eps, bias1, bias2,
+                                     _stream_ptr(self.device)), "adam")

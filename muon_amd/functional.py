@@ -1,0 +1,131 @@
+"""Functional API with the reference's names and argument order (reference muon.py:8-15,
+104-109, 265-291), executed by the gfx950 kernels of libmuon_amd.so."""
+from __future__ import annotations
+
+from collections import OrderedDict
+
+import torch
+
+from . import _lib
+from .engine import AdamGroupEngine, MuonGroupEngine, require_gpu_tensor
+
+_ROUNDINGS = {"reference": True, "fused": False}
+_ENGINE_CACHE: "OrderedDict[tuple, object]" = OrderedDict()
+_ENGINE_CACHE_MAX = 4     # each cached engine holds its bf16 workspace
+
+
+def _cached(key, make):
+    eng = _ENGINE_CACHE.get(key)
+    if eng is None:
+        eng = make()
+        _ENGINE_CACHE[key] = eng
+        while len(_ENGINE_CACHE) > _ENGINE_CACHE_MAX:
+            _ENGINE_CACHE.popitem(last=False)
+    else:
+        _ENGINE_CACHE.move_to_end(key)
+    return eng
+
+
+def clear_engine_cache() -> None:
+    """Drop the workspaces cached by the functional entry points."""
+    _ENGINE_CACHE.clear()
+
+
+def _rounding_flag(rounding: str) -> bool:
+    if rounding not in _ROUNDINGS:
+        raise ValueError(f"rounding must be one of {sorted(_ROUNDINGS)}, got {rounding!r}")
+    return _ROUNDINGS[rounding]
+
+
+def _src_dtype(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _lib.SRC_F32
+    if t.dtype == torch.bfloat16:
+        return _lib.SRC_BF16
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float = 1e-7, *,
+                                rounding: str = "reference") -> torch.Tensor:
+    """Newton-Schulz orthogonalisation of G (reference muon.py:265-291): bf16 result of the
+    shape of G; leading dimensions are a batch.
+
+    rounding="reference" rounds to bf16 wherever the reference's bf16 tensor expression does;
+    "fused" rounds once per stored matrix (closer to the fp32 result).
+    """
+    assert G.ndim >= 2                                     # muon.py:275
+    require_gpu_tensor(G, "G")
+    ref = _rounding_flag(rounding)
+    if G.dtype not in (torch.float32, torch.bfloat16):
+        G = G.float()
+    G = G.contiguous()
+    rows, cols = G.size(-2), G.size(-1)
+    batch = G.numel() // (rows * cols) if rows * cols else 0
+    out = torch.empty(G.shape, dtype=torch.bfloat16, device=G.device)
+    if G.numel() == 0:
+        return out
+    with torch.cuda.device(G.device):
+        eng = _cached(("ns", G.device, rows, cols, batch, int(steps), ref),
+                      lambda: MuonGroupEngine([(rows, cols)] * batch, G.device, int(steps), ref))
+        gsz, osz = rows * cols * G.element_size(), rows * cols * 2
+        eng.run([G.data_ptr() + b * gsz for b in range(batch)], [0] * batch, [0] * batch,
+                [out.data_ptr() + b * osz for b in range(batch)], [1.0] * batch,
+                [_src_dtype(G)] * batch, beta=0.0, nesterov=False, mutate_grad=False,
+                eps=float(epsilon), lr=0.0, weight_decay=0.0)
+    return out
+
+
+def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
+                nesterov: bool = True, ns_steps: int = 5, *, rounding: str = "reference") -> torch.Tensor:
+    """Reference muon.py:8-15.  Updates `momentum` in place, overwrites `grad` with the Nesterov
+    blend (as the reference's grad.lerp_ does) and returns the scaled bf16 orthogonalised update
+    (2-D for 4-D conv filters, else the shape of grad)."""
+    require_gpu_tensor(grad, "grad")
+    require_gpu_tensor(momentum, "momentum")
+    assert grad.ndim >= 2                                  # muon.py:275 via muon.py:13
+    if grad.dtype != torch.float32 or momentum.dtype != torch.float32:
+        raise TypeError("muon_update needs fp32 grad and momentum")
+    if not (grad.is_contiguous() and momentum.is_contiguous()):
+        raise ValueError("muon_update needs contiguous grad and momentum (they are updated in place)")
+    assert grad.shape == momentum.shape
+    ref = _rounding_flag(rounding)
+    if grad.ndim == 4:                                     # muon.py:11-12
+        rows, cols = grad.size(0), grad.numel() // max(grad.size(0), 1)
+        batch, out_shape = 1, (rows, cols)
+    else:
+        rows, cols = grad.size(-2), grad.size(-1)
+        batch, out_shape = (grad.numel() // (rows * cols) if rows * cols else 0), tuple(grad.shape)
+    scale = max(1, grad.size(-2) / grad.size(-1)) ** 0.5   # muon.py:14 (sizes of the un-flattened grad)
+    out = torch.empty(out_shape, dtype=torch.bfloat16, device=grad.device)
+    if grad.numel() == 0:
+        return out
+    with torch.cuda.device(grad.device):
+        eng = _cached(("ns", grad.device, rows, cols, batch, int(ns_steps), ref),
+                      lambda: MuonGroupEngine([(rows, cols)] * batch, grad.device, int(ns_steps), ref))
+        gsz, osz = rows * cols * 4, rows * cols * 2
+        eng.run([grad.data_ptr() + b * gsz for b in range(batch)],
+                [momentum.data_ptr() + b * gsz for b in range(batch)], [0] * batch,
+                [out.data_ptr() + b * osz for b in range(batch)], [scale] * batch,
+                [_lib.SRC_F32] * batch, beta=beta, nesterov=bool(nesterov), mutate_grad=True,
+                eps=1e-7, lr=0.0, weight_decay=0.0)
+    return out
+
+
+def adam_update(grad, buf1, buf2, step, betas, eps) -> torch.Tensor:
+    """Reference muon.py:104-109: updates both moment buffers in place and returns the
+    bias-corrected Adam direction (fp32)."""
+    for name, t in (("grad", grad), ("buf1", buf1), ("buf2", buf2)):
+        require_gpu_tensor(t, name)
+        if t.dtype != torch.float32:
+            raise TypeError("adam_update needs fp32 tensors")
+    if not (buf1.is_contiguous() and buf2.is_contiguous()):
+        raise ValueError("adam_update needs contiguous moment buffers (they are updated in place)")
+    grad = grad.contiguous()
+    out = torch.empty_like(grad)
+    if grad.numel() == 0:
+        return out
+    with torch.cuda.device(grad.device):
+        eng = _cached(("adam", grad.device, grad.numel()), lambda: AdamGroupEngine([grad.numel()], grad.device))
+        eng.run([0], [grad.data_ptr()], [buf1.data_ptr()], [buf2.data_ptr()], [out.data_ptr()],
+                lr=0.0, weight_decay=0.0, betas=betas, eps=float(eps), step=step)
+    return out

@@ -1,0 +1,222 @@
+"""Optimizer classes with the reference's names, constructor signatures, defaults, state keys and
+assertions (reference muon.py:18-70, 73-101, 112-199, 202-260), single-GPU semantics.
+
+Each `step()` issues, per Muon parameter group, a handful of grouped launches over all matrices
+of the group (momentum -> norm -> normalise -> 15 Newton-Schulz GEMM launches -> apply) and one
+fused launch per Adam group; nothing in it synchronises with the host.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .engine import AdamGroupEngine, MuonGroupEngine, require_gpu_tensor
+from .functional import _rounding_flag
+
+NS_STEPS = 5          # the reference classes never pass a step count: muon_update's default rules
+NESTEROV = True       # likewise (muon.py:8)
+
+
+def _world_size() -> int:
+    import torch.distributed as dist
+    return dist.get_world_size() if dist.is_available() and dist.is_initialized() else 1
+
+
+class _MuonBase(torch.optim.Optimizer):
+    """Shared machinery: engine caches and the two per-group update paths."""
+
+    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes):
+        self._reference_rounding = _rounding_flag(ns_rounding)
+        self._mutate_grad = bool(mutate_grad)
+        self._workspace_bytes = workspace_bytes
+        self._muon_engines = {}
+        self._adam_engines = {}
+
+    def __setstate__(self, state):
+        # torch pickles only defaults/state/param_groups; engines (device workspaces and raw
+        # addresses) are rebuilt on the next step.
+        super().__setstate__(state)
+        if not hasattr(self, "_muon_engines"):
+            self._init_runtime("reference", False, None)
+
+    @staticmethod
+    def _check_param(p):
+        require_gpu_tensor(p, "parameter")
+        if p.dtype != torch.float32:
+            raise NotImplementedError(f"muon_amd updates fp32 parameters; got {p.dtype}")
+        if not p.is_contiguous():
+            raise NotImplementedError("muon_amd needs contiguous parameters")
+
+    @staticmethod
+    def _grad_of(p):
+        if p.grad is None:
+            p.grad = torch.zeros_like(p)          # muon.py:91-93 "Force synchronization"
+        g = p.grad
+        if g.dtype != torch.float32 or g.is_sparse:
+            raise NotImplementedError("muon_amd needs dense fp32 gradients")
+        if not g.is_contiguous():
+            g = p.grad = g.contiguous()
+        return g
+
+    def _muon_group_step(self, gi, group):
+        params = [p for p in group["params"] if p.numel() > 0]
+        if not params:
+            return
+        grads, moms, shapes, scales = [], [], [], []
+        for p in params:
+            self._check_param(p)
+            assert p.ndim >= 2                    # muon.py:275 (reached through muon.py:13)
+            g = self._grad_of(p)
+            state = self.state[p]
+            if len(state) == 0:                   # muon.py:95-96
+                state["momentum_buffer"] = torch.zeros_like(p)
+            m = state["momentum_buffer"]
+            if m.dtype != torch.float32 or not m.is_contiguous() or m.device != p.device:
+                raise NotImplementedError("momentum_buffer must be a contiguous fp32 tensor on the parameter's device")
+            if p.ndim == 4:                       # muon.py:11-12
+                rows, cols = p.size(0), p.numel() // p.size(0)
+            elif p.ndim == 2:
+                rows, cols = p.shape
+            else:
+                raise NotImplementedError("muon_amd optimizers take 2-D matrices and 4-D conv filters")
+            shapes.append((rows, cols))
+            scales.append(max(1, p.size(-2) / p.size(-1)) ** 0.5)     # muon.py:14
+            grads.append(g.data_ptr())
+            moms.append(m.data_ptr())
+        device = params[0].device
+        key = (gi, device, tuple(shapes))
+        eng = self._muon_engines.get(key)
+        if eng is None:
+            self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
+            eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes)
+            self._muon_engines[key] = eng
+        n = len(params)
+        with torch.cuda.device(device):
+            eng.run(grads, moms, [p.data_ptr() for p in params], [0] * n, scales, [_lib.SRC_F32] * n,
+                    beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad,
+                    eps=1e-7, lr=group["lr"], weight_decay=group["weight_decay"])
+
+    def _adam_group_step(self, gi, group):
+        by_step = {}
+        for p in group["params"]:
+            self._check_param(p)
+            g = self._grad_of(p)
+            state = self.state[p]
+            if len(state) == 0:                   # muon.py:250-253
+                state["exp_avg"] = torch.zeros_like(p)
+                state["exp_avg_sq"] = torch.zeros_like(p)
+                state["step"] = 0
+            state["step"] += 1                    # muon.py:254
+            if p.numel() > 0:
+                by_step.setdefault(int(state["step"]), []).append((p, g, state))
+        for step, items in by_step.items():
+            device = items[0][0].device
+            key = (gi, device, tuple(id(p) for p, _, _ in items))
+            eng = self._adam_engines.get(key)
+            if eng is None:
+                eng = AdamGroupEngine([p.numel() for p, _, _ in items], device)
+                self._adam_engines[key] = eng
+            with torch.cuda.device(device):
+                eng.run([p.data_ptr() for p, _, _ in items], [g.data_ptr() for _, g, _ in items],
+                        [s["exp_avg"].data_ptr() for _, _, s in items],
+                        [s["exp_avg_sq"].data_ptr() for _, _, s in items], [0] * len(items),
+                        lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"],
+                        eps=group["eps"], step=step)
+
+    @staticmethod
+    def _run_closure(closure):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        return loss
+
+
+class SingleDeviceMuon(_MuonBase):
+    """Muon for one device (reference muon.py:73-101).
+
+    Keyword-only extras (not in the reference): ns_rounding ("reference" | "fused"),
+    mutate_grad (write the Nesterov blend back into p.grad as the reference's in-place lerp does;
+    off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace).
+    """
+
+    def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
+                 mutate_grad=False, workspace_bytes=None):
+        defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
+        super().__init__(params, defaults)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = self._run_closure(closure)
+        for gi, group in enumerate(self.param_groups):
+            self._muon_group_step(gi, group)
+        return loss
+
+
+class Muon(SingleDeviceMuon):
+    """Reference muon.py:18-70 on one GPU: asserts a non-empty list of Parameters and sorts it by
+    size (descending) as the reference does; the cross-rank update sharding is not part of this
+    library, so a process group with more than one rank is refused."""
+
+    def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, **extras):
+        assert isinstance(params, list) and len(params) >= 1 and isinstance(params[0], torch.nn.Parameter)
+        params = sorted(params, key=lambda x: x.size(), reverse=True)      # muon.py:42
+        super().__init__(params, lr=lr, weight_decay=weight_decay, momentum=momentum, **extras)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if _world_size() > 1:
+            raise NotImplementedError("muon_amd.Muon runs on one GPU; sharded updates across ranks are not provided")
+        return super().step(closure)
+
+
+def _fill_aux_adam_groups(param_groups, sort_muon: bool):
+    for group in param_groups:
+        assert "use_muon" in group
+        if group["use_muon"]:
+            if sort_muon:
+                group["params"] = sorted(group["params"], key=lambda x: x.size(), reverse=True)  # muon.py:143
+            group["lr"] = group.get("lr", 0.02)
+            group["momentum"] = group.get("momentum", 0.95)
+            group["weight_decay"] = group.get("weight_decay", 0)
+            assert set(group.keys()) == set(["params", "lr", "momentum", "weight_decay", "use_muon"])
+        else:
+            group["lr"] = group.get("lr", 3e-4)
+            group["betas"] = group.get("betas", (0.9, 0.95))
+            group["eps"] = group.get("eps", 1e-10)
+            group["weight_decay"] = group.get("weight_decay", 0)
+            assert set(group.keys()) == set(["params", "lr", "betas", "eps", "weight_decay", "use_muon"])
+
+
+class SingleDeviceMuonWithAuxAdam(_MuonBase):
+    """Reference muon.py:202-260: Muon for `use_muon=True` groups, Adam for the others."""
+
+    _SORT_MUON = False
+
+    def __init__(self, param_groups, *, ns_rounding="reference", mutate_grad=False, workspace_bytes=None):
+        _fill_aux_adam_groups(param_groups, self._SORT_MUON)
+        super().__init__(param_groups, dict())
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = self._run_closure(closure)
+        for gi, group in enumerate(self.param_groups):
+            if group["use_muon"]:
+                self._muon_group_step(gi, group)
+            else:
+                self._adam_group_step(gi, group)
+        return loss
+
+
+class MuonWithAuxAdam(SingleDeviceMuonWithAuxAdam):
+    """Reference muon.py:112-199 on one GPU (Muon groups sorted by size as the reference does)."""
+
+    _SORT_MUON = True
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if _world_size() > 1:
+            raise NotImplementedError("muon_amd.MuonWithAuxAdam runs on one GPU; sharded updates across ranks are not provided")
+        return super().step(closure)

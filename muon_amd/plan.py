@@ -1,0 +1,261 @@
+"""Host-side planning of the grouped Newton-Schulz launches (pure numpy; no GPU needed).
+
+A *chunk* is a set of matrices that runs through the whole Muon step together: one momentum
+launch, one norm launch, one normalise launch, 3 GEMM launches per Newton-Schulz iteration and
+one apply launch, however many matrices it holds.  Chunks exist only to bound the bf16
+workspace; they share one workspace and run back to back on the stream.
+
+Per matrix (m = min(rows, cols), n = max(rows, cols), padded to the chunk's GEMM tile) the
+workspace holds X (m x n), two copies of X^T (n x m, ping-pong), A, B and c*A (m x m).  The
+un-normalised bf16 update produced by the momentum kernel is parked in the second X^T buffer,
+which the iteration does not touch before the normalise kernel has consumed it.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from functools import lru_cache
+
+import numpy as np
+
+from . import _lib
+
+NS_COEFFS = (3.4445, -4.7750, 2.0315)   # reference muon.py:276
+TILE_EDGE = {0: 128, 1: 256}            # must match muon_amd_gemm_tile()
+EW_BLOCK_ELEMS = 8192                   # must match muon_amd_elementwise_block_elems()
+NT_TILE = 64                            # must match muon_amd_normalize_tile()
+N_XCD = 8                               # workgroups are dealt round-robin to the 8 XCDs
+SUPER_I, SUPER_J = 4, 8                 # output tiles per XCD-resident super-block
+_ALIGN = 256
+
+PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST = range(5)
+
+
+def tile_class_for(m: int) -> int:
+    """256-wide tiles once the short side fills them; 128-wide tiles below that."""
+    return 1 if m >= 1024 else 0
+
+
+def _round_up(x: int, q: int) -> int:
+    return (x + q - 1) // q * q
+
+
+@dataclass
+class MatLayout:
+    index: int            # position in the caller's matrix list
+    rows: int
+    cols: int
+    m: int
+    n: int
+    mp: int
+    np_: int
+    wide: bool            # rows <= cols: X is the matrix itself; else X is its transpose
+    off: dict = field(default_factory=dict)   # byte offsets of X, XT0, XT1, A, B, CA
+
+    @property
+    def rows_p(self) -> int:
+        return self.mp if self.wide else self.np_
+
+    @property
+    def cols_p(self) -> int:
+        return self.np_ if self.wide else self.mp
+
+    @property
+    def numel(self) -> int:
+        return self.rows * self.cols
+
+
+def matrix_workspace_bytes(rows: int, cols: int, tile: int) -> int:
+    m, n = min(rows, cols), max(rows, cols)
+    mp, np_ = _round_up(m, tile), _round_up(n, tile)
+    return 3 * _round_up(mp * np_ * 2, _ALIGN) + 3 * _round_up(mp * mp * 2, _ALIGN)
+
+
+@lru_cache(maxsize=256)
+def _tile_order(mt: int, nt: int, sym: bool):
+    """Tiles of an mt x nt grid (upper triangle if sym) in super-block order."""
+    ti, tj = [], []
+    for bi in range(0, mt, SUPER_I):
+        for bj in range(0, nt, SUPER_J):
+            for i in range(bi, min(bi + SUPER_I, mt)):
+                for j in range(bj, min(bj + SUPER_J, nt)):
+                    if sym and j < i:
+                        continue
+                    ti.append(i)
+                    tj.append(j)
+    return np.asarray(ti, dtype=np.int32), np.asarray(tj, dtype=np.int32)
+
+
+def xcd_permutation(njobs: int) -> np.ndarray:
+    """physical block b runs logical job perm[b]: XCD x = b % 8 walks a contiguous logical range,
+    so the 32 workgroups resident on one XCD share operand panels in that XCD's L2."""
+    seg = -(-njobs // N_XCD)
+    idx = np.arange(N_XCD * seg, dtype=np.int64).reshape(N_XCD, seg).T.reshape(-1)
+    return idx[idx < njobs]
+
+
+class ChunkPlan:
+    """Layout, descriptor tables and tile job lists of one chunk."""
+
+    def __init__(self, mats, tile_class: int, steps: int, reference_rounding: bool):
+        # mats: list of (index, rows, cols)
+        self.tile_class = tile_class
+        self.tile = TILE_EDGE[tile_class]
+        self.steps = steps
+        self.reference_rounding = reference_rounding
+        T = self.tile
+        self.layouts: list[MatLayout] = []
+        off = 0
+        for index, rows, cols in mats:
+            m, n = min(rows, cols), max(rows, cols)
+            lay = MatLayout(index, rows, cols, m, n, _round_up(m, T), _round_up(n, T), rows <= cols)
+            xb = _round_up(lay.mp * lay.np_ * 2, _ALIGN)
+            ab = _round_up(lay.mp * lay.mp * 2, _ALIGN)
+            for name, nbytes in (("X", xb), ("XT0", xb), ("XT1", xb), ("A", ab), ("B", ab), ("CA", ab)):
+                lay.off[name] = off
+                off += nbytes
+            self.layouts.append(lay)
+        self.nmat = len(self.layouts)
+        # elementwise block prefix (momentum / apply) and normalise tile prefix
+        nblk = [-(-lay.numel // EW_BLOCK_ELEMS) for lay in self.layouts]
+        self.block_prefix = np.concatenate([[0], np.cumsum(nblk)]).astype(np.int32)
+        self.nblocks = int(self.block_prefix[-1])
+        ntile = [(lay.rows_p // NT_TILE) * (lay.cols_p // NT_TILE) for lay in self.layouts]
+        self.tile_prefix = np.concatenate([[0], np.cumsum(ntile)]).astype(np.int32)
+        self.ntiles = int(self.tile_prefix[-1])
+        # scalars at the tail of the workspace
+        self.off_partials = off
+        off += _round_up(self.nblocks * 4, _ALIGN)
+        self.off_denoms = off
+        off += _round_up(self.nmat * 4, _ALIGN)
+        self.workspace_bytes = off
+        self.sym_jobs = self._jobs(sym=True)
+        self.full_jobs = self._jobs(sym=False)
+
+    # ---- tile job lists -----------------------------------------------------------------
+    def _jobs(self, sym: bool) -> np.ndarray:
+        T = self.tile
+        parts = []
+        for k, lay in enumerate(self.layouts):
+            mt = lay.mp // T
+            nt = mt if sym else lay.np_ // T
+            ti, tj = _tile_order(mt, nt, sym)
+            j = np.zeros(len(ti), dtype=_lib.TILE_JOB)
+            j["desc"] = k
+            j["i0"] = ti * T
+            j["j0"] = tj * T
+            j["diag"] = (ti == tj).astype(np.int32) if sym else 0
+            parts.append(j)
+        logical = np.concatenate(parts)
+        return np.ascontiguousarray(logical[xcd_permutation(len(logical))])
+
+    # ---- descriptor tables -----------------------------------------------------------------
+    def result_buffer(self, lay: MatLayout) -> str:
+        if self.steps == 0:
+            return "X" if lay.wide else "XT0"
+        return "X" if lay.wide else ("XT1" if self.steps % 2 else "XT0")
+
+    def gemm_descs(self, base: int) -> np.ndarray:
+        """[5, nmat] MuonGemmDesc table for a workspace at device address `base`."""
+        d = np.zeros((5, self.nmat), dtype=_lib.GEMM_DESC)
+        for k, lay in enumerate(self.layouts):
+            p = {name: base + o for name, o in lay.off.items()}
+            mp, np_ = lay.mp, lay.np_
+            s = d[PH_SYRK, k]
+            s["P"] = s["Q"] = p["X"]
+            s["ldp"] = s["ldq"] = np_
+            s["K"] = np_
+            s["C"] = s["CT"] = p["A"]
+            if self.reference_rounding:
+                s["C2"] = s["C2T"] = p["CA"]
+            s["ldc"] = s["ldct"] = mp
+            s["rows"] = s["colsn"] = mp
+            q = d[PH_POLY, k]
+            q["P"] = p["CA"] if self.reference_rounding else p["A"]
+            q["Q"] = q["D"] = p["A"]
+            q["ldp"] = q["ldq"] = q["ldd"] = mp
+            q["K"] = mp
+            q["C"] = q["CT"] = p["B"]
+            q["ldc"] = q["ldct"] = mp
+            q["rows"] = q["colsn"] = mp
+            for ph, src, dst in ((PH_UPD_EVEN, "XT0", "XT1"), (PH_UPD_ODD, "XT1", "XT0")):
+                u = d[ph, k]
+                u["P"] = p["B"]
+                u["ldp"] = mp
+                u["Q"] = p[src]
+                u["ldq"] = mp
+                u["K"] = mp
+                u["D"] = u["C"] = p["X"]
+                u["ldd"] = u["ldc"] = np_
+                u["CT"] = p[dst]
+                u["ldct"] = mp
+                u["rows"] = mp
+                u["colsn"] = np_
+            last = d[PH_UPD_LAST, k]
+            if self.steps > 0:
+                last_src = d[PH_UPD_EVEN if (self.steps - 1) % 2 == 0 else PH_UPD_ODD, k]
+                for name in _lib.GEMM_DESC.names:
+                    last[name] = last_src[name]
+                if lay.wide:
+                    last["CT"] = 0
+                else:
+                    last["C"] = 0
+            else:
+                for name in _lib.GEMM_DESC.names:   # never launched; keep it well formed
+                    last[name] = d[PH_UPD_EVEN, k][name]
+        return d
+
+    def mat_descs(self, base: int) -> np.ndarray:
+        """MuonMatDesc table with the workspace fields filled; tensor pointers are left zero."""
+        d = np.zeros(self.nmat, dtype=_lib.MAT_DESC)
+        for k, lay in enumerate(self.layouts):
+            p = {name: base + o for name, o in lay.off.items()}
+            r = d[k]
+            r["u"] = p["XT1"]
+            r["direct"] = p["X"] if lay.wide else p["XT0"]
+            r["transp"] = p["XT0"] if lay.wide else p["X"]
+            r["result"] = p[self.result_buffer(lay)]
+            r["partials"] = base + self.off_partials
+            r["denom"] = base + self.off_denoms + 4 * k
+            r["rows"], r["cols"] = lay.rows, lay.cols
+            r["rows_p"], r["cols_p"] = lay.rows_p, lay.cols_p
+            r["part_begin"] = self.block_prefix[k]
+            r["part_end"] = self.block_prefix[k + 1]
+            r["scale"] = 1.0
+        return d
+
+    def phase_scalars(self, phase: int):
+        """(alpha, beta, gamma) of the GEMM epilogue for a phase."""
+        a, b, c = NS_COEFFS
+        if phase == PH_SYRK:
+            return 1.0, 0.0, c
+        if phase == PH_POLY:
+            return (1.0, b, 0.0) if self.reference_rounding else (c, b, 0.0)
+        return 1.0, a, 0.0
+
+
+def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int):
+    """Split matrices [(rows, cols), ...] into chunks of one tile class each whose workspace stays
+    under `workspace_cap` bytes (a single matrix larger than the cap gets a chunk of its own).
+    Same-shape matrices are kept together so that their tiles batch into full waves of the GPU."""
+    order = sorted(range(len(shapes)),
+                   key=lambda i: (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]),
+                                  -shapes[i][0], i))
+    chunks, cur, cur_bytes, cur_class = [], [], 0, None
+    for i in order:
+        rows, cols = shapes[i]
+        tc = tile_class_for(min(rows, cols))
+        need = matrix_workspace_bytes(rows, cols, TILE_EDGE[tc])
+        if cur and (tc != cur_class or cur_bytes + need > workspace_cap):
+            chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding))
+            cur, cur_bytes = [], 0
+        cur.append((i, rows, cols))
+        cur_bytes += need
+        cur_class = tc
+    if cur:
+        chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding))
+    return chunks
+
+
+def adam_block_prefix(numels) -> np.ndarray:
+    nblk = [-(-int(n) // EW_BLOCK_ELEMS) for n in numels]
+    return np.concatenate([[0], np.cumsum(nblk)]).astype(np.int32)

@@ -1,0 +1,243 @@
+"""CPU oracle for the Muon optimizer step.  TEST INFRASTRUCTURE -- not product code.
+
+Only the test-suite, the smoke check and the benchmark's CPU-baseline leg may import this
+module; the shipped package never does.  Everything here runs on the CPU with plain
+torch / numpy operations and restates, line by line, the algorithm of the reference
+implementation (all citations are into /root/reference/muon.py):
+
+  ns5_bf16 / ns5_fp32        muon.py:265-291  (the Newton-Schulz specification: Frobenius
+                             pre-scale, `steps` quintic iterations with a, b, c =
+                             3.4445, -4.7750, 2.0315, transpose-if-tall, bf16 storage)
+  ns5_fp64_closed_form       the same map written through the SVD in float64:
+                             U diag(p^steps(sigma / ||G||_F)) V^T, p(x) = a x + b x^3 + c x^5
+  muon_update                muon.py:8-15
+  adam_update                muon.py:104-109
+  OracleSingleDeviceMuon     muon.py:73-101
+  OracleSingleDeviceMuonWithAuxAdam   muon.py:202-260
+
+What pins each function (the reference ships no tests, golden vectors or fixtures):
+  * ns5_fp32      -- against ns5_fp64_closed_form (independent derivation through the SVD),
+                     a triple-loop float64 brute force on tiny matrices, and the invariants
+                     NS(G^T)=NS(G)^T, NS(alpha G)=NS(G), NS(Q1 G Q2)=Q1 NS(G) Q2, NS(0)=0,
+                     NS(diag d)=diag(p^5(d/||d||)), NS(Q)=p^5(1/sqrt(m)) Q.
+  * ns5_bf16      -- same code path as ns5_fp32 with the bf16 casts of muon.py:277; pinned to
+                     ns5_fp32 within bf16 rounding noise and to the same invariants.
+  * muon_update   -- first-step closed form (zero momentum => update = NS(g) because the
+                     Nesterov blend is (1-beta^2) g and NS is scale invariant), float64
+                     recurrences for several steps, the conv-shape aspect-ratio rule.
+  * adam_update   -- equals torch.optim.AdamW step for step; first-step closed form g/(|g|+eps).
+  * step classes  -- behavioural unit tests written from the cited lines.
+No function here is "parity unpinned".
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+NS_COEFFS = (3.4445, -4.7750, 2.0315)  # muon.py:276
+
+
+# --------------------------------------------------------------------------------------
+# Newton-Schulz (muon.py:265-291)
+# --------------------------------------------------------------------------------------
+def _ns5(G: torch.Tensor, steps: int, eps: float, work_dtype: torch.dtype) -> torch.Tensor:
+    assert G.ndim >= 2                                    # muon.py:275
+    a, b, c = NS_COEFFS                                   # muon.py:276
+    X = G.to(work_dtype)                                  # muon.py:277 (bf16 in the reference)
+    tall = G.size(-2) > G.size(-1)
+    if tall:                                              # muon.py:278-279
+        X = X.mT
+    X = X / (X.norm(dim=(-2, -1), keepdim=True) + eps)    # muon.py:282
+    for _ in range(steps):                                # muon.py:284
+        A = X @ X.mT                                      # muon.py:285
+        B = b * A + c * A @ A                             # muon.py:286  ((c*A) @ A)
+        X = a * X + B @ X                                 # muon.py:287
+    if tall:                                              # muon.py:289-290
+        X = X.mT
+    return X
+
+
+def ns5_bf16(G: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.Tensor:
+    """The reference bf16 result: muon.py:265-291 run with torch CPU bf16 arithmetic."""
+    return _ns5(G, steps, eps, torch.bfloat16)
+
+
+def ns5_fp32(G: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.Tensor:
+    """The fp32 oracle: same sequence without the bf16 cast."""
+    return _ns5(G.float(), steps, eps, torch.float32)
+
+
+def ns_poly(x, steps: int = 5):
+    """p^steps(x) with p(x) = a x + b x^3 + c x^5, the scalar map NS applies to singular values."""
+    a, b, c = NS_COEFFS
+    x = np.asarray(x, dtype=np.float64)
+    for _ in range(steps):
+        x2 = x * x
+        x = x * (a + x2 * (b + c * x2))
+    return x
+
+
+def ns5_fp64_closed_form(G, steps: int = 5, eps: float = 1e-7) -> np.ndarray:
+    """U diag(p^steps(sigma/(||G||_F+eps))) V^T in float64; 2-D input only."""
+    G = np.asarray(G.detach().double().cpu().numpy() if isinstance(G, torch.Tensor) else G,
+                   dtype=np.float64)
+    assert G.ndim == 2
+    U, s, Vt = np.linalg.svd(G, full_matrices=False)
+    fro = np.sqrt((s * s).sum())
+    return (U * ns_poly(s / (fro + eps), steps)) @ Vt
+
+
+# --------------------------------------------------------------------------------------
+# Update rules
+# --------------------------------------------------------------------------------------
+def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
+                nesterov: bool = True, ns_steps: int = 5) -> torch.Tensor:
+    """muon.py:8-15.  Mutates `momentum` and (with nesterov) `grad` exactly as the reference."""
+    momentum.lerp_(grad, 1 - beta)                                        # muon.py:9
+    update = grad.lerp_(momentum, beta) if nesterov else momentum         # muon.py:10
+    if update.ndim == 4:                                                  # muon.py:11-12
+        update = update.view(len(update), -1)
+    update = ns5_bf16(update, ns_steps)                                   # muon.py:13
+    update *= max(1, grad.size(-2) / grad.size(-1)) ** 0.5                # muon.py:14
+    return update
+
+
+def adam_update(grad, buf1, buf2, step, betas, eps):
+    """muon.py:104-109."""
+    buf1.lerp_(grad, 1 - betas[0])                       # muon.py:105
+    buf2.lerp_(grad.square(), 1 - betas[1])              # muon.py:106
+    buf1c = buf1 / (1 - betas[0] ** step)                # muon.py:107
+    buf2c = buf2 / (1 - betas[1] ** step)                # muon.py:108
+    return buf1c / (buf2c.sqrt() + eps)                  # muon.py:109
+
+
+# --------------------------------------------------------------------------------------
+# Optimizer classes (single-device semantics)
+# --------------------------------------------------------------------------------------
+class OracleSingleDeviceMuon(torch.optim.Optimizer):
+    """muon.py:73-101."""
+
+    def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95):
+        defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
+        super().__init__(params, defaults)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for group in self.param_groups:
+            for p in group["params"]:
+                _muon_param_step(self, p, group)
+        return loss
+
+
+def _muon_param_step(opt, p, group):
+    if p.grad is None:                                                     # muon.py:91-93
+        p.grad = torch.zeros_like(p)
+    state = opt.state[p]
+    if len(state) == 0:                                                    # muon.py:95-96
+        state["momentum_buffer"] = torch.zeros_like(p)
+    update = muon_update(p.grad, state["momentum_buffer"], beta=group["momentum"])  # :97
+    p.mul_(1 - group["lr"] * group["weight_decay"])                        # muon.py:98
+    p.add_(update.reshape(p.shape), alpha=-group["lr"])                    # muon.py:99
+
+
+def _adam_param_step(opt, p, group):
+    if p.grad is None:                                                     # muon.py:246-248
+        p.grad = torch.zeros_like(p)
+    state = opt.state[p]
+    if len(state) == 0:                                                    # muon.py:250-253
+        state["exp_avg"] = torch.zeros_like(p)
+        state["exp_avg_sq"] = torch.zeros_like(p)
+        state["step"] = 0
+    state["step"] += 1                                                     # muon.py:254
+    update = adam_update(p.grad, state["exp_avg"], state["exp_avg_sq"],
+                         state["step"], group["betas"], group["eps"])      # muon.py:255-256
+    p.mul_(1 - group["lr"] * group["weight_decay"])                        # muon.py:257
+    p.add_(update, alpha=-group["lr"])                                     # muon.py:258
+
+
+class OracleSingleDeviceMuonWithAuxAdam(torch.optim.Optimizer):
+    """muon.py:202-260."""
+
+    def __init__(self, param_groups):
+        for group in param_groups:
+            assert "use_muon" in group
+            if group["use_muon"]:
+                group["lr"] = group.get("lr", 0.02)
+                group["momentum"] = group.get("momentum", 0.95)
+                group["weight_decay"] = group.get("weight_decay", 0)
+                assert set(group.keys()) == {"params", "lr", "momentum", "weight_decay", "use_muon"}
+            else:
+                group["lr"] = group.get("lr", 3e-4)
+                group["betas"] = group.get("betas", (0.9, 0.95))
+                group["eps"] = group.get("eps", 1e-10)
+                group["weight_decay"] = group.get("weight_decay", 0)
+                assert set(group.keys()) == {"params", "lr", "betas", "eps", "weight_decay", "use_muon"}
+        super().__init__(param_groups, dict())
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        for group in self.param_groups:
+            if group["use_muon"]:
+                for p in group["params"]:
+                    _muon_param_step(self, p, group)
+            else:
+                for p in group["params"]:
+                    _adam_param_step(self, p, group)
+        return loss
+
+
+# --------------------------------------------------------------------------------------
+# Helpers used by tests
+# --------------------------------------------------------------------------------------
+def rel_fro(x, ref) -> float:
+    """Relative Frobenius error ||x - ref||_F / ||ref||_F computed in float64."""
+    x = x.detach().double().cpu() if isinstance(x, torch.Tensor) else torch.as_tensor(np.asarray(x)).double()
+    ref = ref.detach().double().cpu() if isinstance(ref, torch.Tensor) else torch.as_tensor(np.asarray(ref)).double()
+    den = ref.norm().item()
+    num = (x - ref).norm().item()
+    return num / den if den > 0 else num
+
+
+def matmul_brute_force(A, B):
+    """Textbook triple loop in Python floats (float64); tiny matrices only."""
+    n, k = len(A), len(A[0])
+    k2, m = len(B), len(B[0])
+    assert k == k2
+    C = [[0.0] * m for _ in range(n)]
+    for i in range(n):
+        for j in range(m):
+            s = 0.0
+            for t in range(k):
+                s += A[i][t] * B[t][j]
+            C[i][j] = s
+    return C
+
+
+def ns5_brute_force(G_rows, steps: int = 5, eps: float = 1e-7):
+    """muon.py:278-290 with every product a triple loop; G_rows: list of lists (2-D)."""
+    a, b, c = NS_COEFFS
+    r, cc = len(G_rows), len(G_rows[0])
+    X = [list(map(float, row)) for row in G_rows]
+    tall = r > cc
+    T = lambda M: [list(col) for col in zip(*M)]
+    if tall:
+        X = T(X)
+    fro = sum(v * v for row in X for v in row) ** 0.5
+    X = [[v / (fro + eps) for v in row] for row in X]
+    for _ in range(steps):
+        A = matmul_brute_force(X, T(X))
+        AA = matmul_brute_force(A, A)
+        B = [[b * A[i][j] + c * AA[i][j] for j in range(len(A))] for i in range(len(A))]
+        BX = matmul_brute_force(B, X)
+        X = [[a * X[i][j] + BX[i][j] for j in range(len(X[0]))] for i in range(len(X))]
+    if tall:
+        X = T(X)
+    return X
