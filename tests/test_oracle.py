@@ -1,0 +1,245 @@
+"""Pins the CPU oracle (oracle/muon_oracle.py) without the reference being importable: closed
+forms, brute force, invariants and library special cases chosen so that a dropped term, a wrong
+sign/index or a transposed operand fails at least one of them."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import muon_oracle as O
+
+A_, B_, C_ = O.NS_COEFFS
+
+
+# ------------------------------------------------------------------------------------------
+# scalar map
+# ------------------------------------------------------------------------------------------
+def test_coefficients_and_scalar_map_facts():
+    assert O.NS_COEFFS == (3.4445, -4.7750, 2.0315)          # muon.py:276
+    p1 = A_ + B_ + C_
+    assert abs(p1 - 0.7010) < 1e-12
+    assert abs(O.ns_poly(1.0, 1) - p1) < 1e-12
+    assert abs(O.ns_poly(1.0, 5) - 0.69644) < 1e-4
+    x = np.linspace(0.005, 1.0, 20001)
+    y = O.ns_poly(x, 5)
+    assert 0.68 < y.min() < 0.69 and 1.15 < y.max() < 1.16
+    # slope at zero after five steps is a^5
+    assert abs(O.ns_poly(1e-9, 5) / 1e-9 - A_ ** 5) < 1e-3
+    assert abs(A_ ** 5 - 484.876) < 1e-2
+
+
+# ------------------------------------------------------------------------------------------
+# Newton-Schulz: closed form, brute force, invariants
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(8, 8), (6, 17), (17, 6), (32, 96), (96, 32), (3, 4)])
+def test_ns_fp32_matches_fp64_svd_closed_form(shape):
+    torch.manual_seed(hash(shape) % 1000)
+    G = torch.randn(*shape, dtype=torch.float64)
+    got = O._ns5(G, 5, 1e-7, torch.float64).numpy()
+    want = O.ns5_fp64_closed_form(G)
+    np.testing.assert_allclose(got, want, rtol=0, atol=1e-9)
+    assert O.rel_fro(O.ns5_fp32(G.float()), want) < 2e-4
+
+
+@pytest.mark.parametrize("shape", [(3, 5), (5, 3), (4, 4), (2, 7)])
+def test_ns_matches_triple_loop_brute_force(shape):
+    torch.manual_seed(7)
+    G = torch.randn(*shape, dtype=torch.float64)
+    brute = np.array(O.ns5_brute_force(G.tolist()))
+    np.testing.assert_allclose(O._ns5(G, 5, 1e-7, torch.float64).numpy(), brute, atol=1e-10)
+    np.testing.assert_allclose(O.ns5_fp64_closed_form(G), brute, atol=1e-9)
+
+
+@pytest.mark.parametrize("steps", [0, 1, 2, 5])
+def test_ns_step_count(steps):
+    torch.manual_seed(3)
+    G = torch.randn(5, 9, dtype=torch.float64)
+    np.testing.assert_allclose(O._ns5(G, steps, 1e-7, torch.float64).numpy(),
+                               O.ns5_fp64_closed_form(G, steps), atol=1e-10)
+    if steps == 0:   # just the Frobenius normalisation
+        np.testing.assert_allclose(O._ns5(G, 0, 1e-7, torch.float64).numpy(),
+                                   (G / (G.norm() + 1e-7)).numpy(), atol=1e-15)
+
+
+def test_ns_transpose_rule():
+    # muon.py:278-279, 289-290: a tall input is iterated as its transpose, so NS(G^T) == NS(G)^T
+    # up to the summation order of the matrix products (strided vs contiguous operands).
+    torch.manual_seed(11)
+    G = torch.randn(40, 24, dtype=torch.float64)
+    a, b = O._ns5(G.mT.contiguous(), 5, 1e-7, torch.float64), O._ns5(G, 5, 1e-7, torch.float64).mT
+    assert O.rel_fro(a, b) < 1e-12
+    assert O.rel_fro(O.ns5_fp32(G.float().mT.contiguous()), O.ns5_fp32(G.float()).mT) < 1e-4
+    assert O.rel_fro(O.ns5_bf16(G.float().mT.contiguous()), O.ns5_bf16(G.float()).mT) < 2e-2
+    sq = torch.randn(16, 16, dtype=torch.float64)   # square is not transposed (strict >) but the map commutes
+    assert O.rel_fro(O._ns5(sq.mT.contiguous(), 5, 0.0, torch.float64), O._ns5(sq, 5, 0.0, torch.float64).mT) < 1e-10
+
+
+def test_ns_scale_and_orthogonal_invariance():
+    torch.manual_seed(5)
+    G = torch.randn(12, 30, dtype=torch.float64)
+    base = O._ns5(G, 5, 0.0, torch.float64)
+    assert O.rel_fro(O._ns5(G * 37.5, 5, 0.0, torch.float64), base) < 1e-12
+    Q1, _ = torch.linalg.qr(torch.randn(12, 12, dtype=torch.float64))
+    Q2, _ = torch.linalg.qr(torch.randn(30, 30, dtype=torch.float64))
+    assert O.rel_fro(O._ns5(Q1 @ G @ Q2, 5, 0.0, torch.float64), Q1 @ base @ Q2) < 1e-10
+
+
+def test_ns_special_inputs():
+    assert torch.equal(O.ns5_fp32(torch.zeros(4, 6)), torch.zeros(4, 6))        # eps keeps 0/0 finite
+    assert torch.equal(O.ns5_bf16(torch.zeros(6, 4)).float(), torch.zeros(6, 4))
+    d = torch.tensor([3.0, 1.0, 0.5, 0.25], dtype=torch.float64)
+    got = O._ns5(torch.diag(d), 5, 0.0, torch.float64)
+    np.testing.assert_allclose(got.numpy(), np.diag(O.ns_poly((d / d.norm()).numpy(), 5)), atol=1e-12)
+    Q, _ = torch.linalg.qr(torch.randn(9, 9, dtype=torch.float64))
+    np.testing.assert_allclose(O._ns5(Q, 5, 0.0, torch.float64).numpy(),
+                               (O.ns_poly(1 / 3.0, 5) * Q).numpy(), atol=1e-10)
+
+
+def test_ns_batched_equals_per_matrix():
+    torch.manual_seed(2)
+    G = torch.randn(3, 10, 14)
+    out = O.ns5_bf16(G)
+    for b in range(3):
+        assert torch.equal(out[b], O.ns5_bf16(G[b]))
+    assert out.dtype == torch.bfloat16 and out.shape == G.shape          # muon.py:277
+
+
+def test_ns_bf16_tracks_fp32_and_singular_values_land_in_band():
+    torch.manual_seed(9)
+    G = torch.randn(128, 384) * 1e-3
+    rb, rf = O.ns5_bf16(G).float(), O.ns5_fp32(G)
+    assert O.rel_fro(rb, rf) < 4e-2
+    s = torch.linalg.svdvals(rf.double())
+    assert s.min() > 0.66 and s.max() < 1.17
+
+
+# ------------------------------------------------------------------------------------------
+# muon_update
+# ------------------------------------------------------------------------------------------
+def test_muon_update_first_step_closed_form():
+    torch.manual_seed(4)
+    g = torch.randn(20, 30) * 1e-3
+    g0 = g.clone()
+    mom = torch.zeros_like(g)
+    upd = O.muon_update(g, mom, beta=0.95)
+    # zero momentum: m = (1-b) g, blend = (1-b) g + b (1-b) g = (1-b^2) g; NS is scale invariant
+    np.testing.assert_allclose(mom.numpy(), (0.05 * g0.double()).float().numpy(), rtol=1e-6)
+    np.testing.assert_allclose(g.numpy(), ((1 - 0.95 ** 2) * g0.double()).float().numpy(), rtol=2e-6)
+    assert upd.dtype == torch.bfloat16
+    assert O.rel_fro(upd, O.ns5_fp64_closed_form(g0)) < 4e-2
+
+
+def test_muon_update_fp64_recurrence_and_no_nesterov():
+    torch.manual_seed(6)
+    mom = torch.zeros(8, 12)
+    m64 = np.zeros((8, 12))
+    for _ in range(4):
+        g = torch.randn(8, 12)
+        g64 = g.double().numpy()
+        m64 = m64 + 0.05 * (g64 - m64)
+        u64 = 0.05 * g64 + 0.95 * m64
+        upd = O.muon_update(g, mom, beta=0.95, nesterov=True)
+        np.testing.assert_allclose(mom.numpy(), m64, rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(g.numpy(), u64, rtol=1e-5, atol=1e-7)
+        assert O.rel_fro(upd, O.ns5_fp64_closed_form(u64)) < 8e-2   # bf16 noise on a tiny matrix
+    g = torch.randn(8, 12)
+    g_before = g.clone()
+    upd = O.muon_update(g, mom, beta=0.9, nesterov=False)
+    assert torch.equal(g, g_before)                       # only the nesterov branch writes grad
+    assert O.rel_fro(upd, O.ns5_fp64_closed_form(mom)) < 8e-2
+
+
+@pytest.mark.parametrize("shape,scale", [((30, 10), math.sqrt(3.0)), ((10, 30), 1.0),
+                                          ((16, 4, 3, 3), 1.0), ((8, 2, 4, 2), math.sqrt(2.0))])
+def test_muon_update_aspect_scale_uses_unflattened_sizes(shape, scale):
+    torch.manual_seed(8)
+    g = torch.randn(*shape)
+    flat = g.reshape(shape[0], -1).clone()
+    upd = O.muon_update(g, torch.zeros_like(g), beta=0.0, nesterov=False)   # beta=0: momentum == grad
+    want = O.ns5_bf16(flat)
+    want = (want.float() * scale).bfloat16() if scale != 1.0 else want
+    assert upd.shape == flat.shape                       # conv filters come back 2-D (muon.py:11-12)
+    assert torch.equal(upd, want)
+
+
+# ------------------------------------------------------------------------------------------
+# adam_update
+# ------------------------------------------------------------------------------------------
+def test_adam_update_first_step_closed_form():
+    g = torch.tensor([1e-3, -2.0, 0.5, 0.0])
+    m, v = torch.zeros(4), torch.zeros(4)
+    upd = O.adam_update(g, m, v, 1, (0.9, 0.95), 1e-10)
+    np.testing.assert_allclose(upd.numpy(), (g / (g.abs() + 1e-10)).numpy(), rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(m.numpy(), 0.1 * g.numpy(), rtol=1e-6)
+    np.testing.assert_allclose(v.numpy(), 0.05 * g.numpy() ** 2, rtol=1e-6)
+
+
+def test_adam_branch_equals_torch_adamw():
+    torch.manual_seed(10)
+    p1 = torch.nn.Parameter(torch.randn(7, 5))
+    p2 = torch.nn.Parameter(p1.detach().clone())
+    o1 = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p1], use_muon=False, lr=1e-2, betas=(0.9, 0.95),
+                                                   eps=1e-10, weight_decay=0.1)])
+    o2 = torch.optim.AdamW([p2], lr=1e-2, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.1)
+    for _ in range(10):
+        g = torch.randn(7, 5)
+        p1.grad, p2.grad = g.clone(), g.clone()
+        o1.step()
+        o2.step()
+    np.testing.assert_allclose(p1.detach().numpy(), p2.detach().numpy(), rtol=1e-5, atol=1e-7)
+
+
+# ------------------------------------------------------------------------------------------
+# step classes
+# ------------------------------------------------------------------------------------------
+def test_single_device_muon_config1_shape_collapses_to_ns_of_grad():
+    torch.manual_seed(1)
+    p = torch.nn.Parameter(torch.randn(48, 192) * 0.02)
+    p0 = p.detach().clone()
+    g = torch.randn(48, 192) * 1e-3
+    p.grad = g.clone()
+    opt = O.OracleSingleDeviceMuon([p], lr=0.02, weight_decay=0.01, momentum=0.95)
+    opt.step()
+    want = p0.double() * (1 - 0.02 * 0.01) - 0.02 * torch.from_numpy(O.ns5_fp64_closed_form(g))
+    assert O.rel_fro(p.detach(), want) < 5e-3    # bf16 NS noise (3e-2) on an update of ~7% of |p|
+    assert set(opt.state[p].keys()) == {"momentum_buffer"}
+
+
+def test_step_classes_behaviour():
+    p = torch.nn.Parameter(torch.ones(4, 6))
+    q = torch.nn.Parameter(torch.ones(5))
+    opt = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=True, weight_decay=0.5),
+                                               dict(params=[q], use_muon=False, weight_decay=0.5)])
+    assert opt.param_groups[0]["lr"] == 0.02 and opt.param_groups[0]["momentum"] == 0.95
+    assert opt.param_groups[1]["lr"] == 3e-4 and opt.param_groups[1]["betas"] == (0.9, 0.95)
+    assert opt.param_groups[1]["eps"] == 1e-10
+    calls = []
+    loss = opt.step(lambda: calls.append(1) or torch.tensor(3.0))
+    assert loss.item() == 3.0 and calls == [1]
+    # grad None -> zeros, parameter still decayed (muon.py:91-93, 98)
+    assert p.grad is not None and torch.count_nonzero(p.grad) == 0
+    np.testing.assert_allclose(p.detach().numpy(), np.full((4, 6), 1 - 0.02 * 0.5), rtol=1e-6)
+    np.testing.assert_allclose(q.detach().numpy(), np.full(5, 1 - 3e-4 * 0.5), rtol=1e-6)
+    assert set(opt.state[q].keys()) == {"exp_avg", "exp_avg_sq", "step"} and opt.state[q]["step"] == 1
+    with pytest.raises(AssertionError):
+        O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=True, betas=(0.9, 0.9))])
+    with pytest.raises(AssertionError):
+        O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p])])
+
+
+# ------------------------------------------------------------------------------------------
+# golden fixtures are what the oracle produces (guards against silent drift of either)
+# ------------------------------------------------------------------------------------------
+def test_oracle_reproduces_golden_fixtures(golden_dir):
+    z = np.load(os.path.join(golden_dir, "ns_golden.npz"))
+    names = sorted({k.split("/")[0] for k in z.files})
+    assert len(names) >= 6
+    for n in names:
+        G = torch.from_numpy(z[n + "/in"])
+        got = O.ns5_bf16(G).contiguous().view(torch.int16).numpy().astype(np.uint16)
+        assert np.array_equal(got, z[n + "/bf16"]), n
+        np.testing.assert_allclose(O.ns5_fp32(G).numpy(), z[n + "/fp32"], rtol=1e-6, atol=1e-7)
+        if G.ndim == 2:
+            assert O.rel_fro(z[n + "/fp32"], z[n + "/fp64_closed_form"]) < 2e-4
