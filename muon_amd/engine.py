@@ -18,6 +18,24 @@ def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
             "CPU implementation")
 
 
+# When set to a list, every launch is bracketed by a pair of HIP events recorded on the stream it
+# runs on, and (label, algorithmic work, start, stop) is appended.  Work is flops for the GEMM
+# launches (the minimum given symmetry, on the unpadded sizes) and bytes for the others.
+PROFILE = None
+
+
+def _launch(label, work, call):
+    if PROFILE is None:
+        call()
+        return
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    call()
+    e1.record()
+    PROFILE.append((label, work, e0, e1))
+
+
 def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -88,20 +106,33 @@ class _ChunkRuntime:
         s = _stream_ptr(self.device)
         flags = _lib.ROUND_REFERENCE if c.reference_rounding else _lib.ROUND_FUSED
         mats = self.mat_dev.data_ptr()
-        _lib.check(lib.muon_amd_momentum(mats, self.block_prefix_ptr, c.nmat, c.nblocks,
-                                         one_minus_beta, beta, int(nesterov), int(mutate_grad), s), "momentum")
-        _lib.check(lib.muon_amd_norm_finalize(mats, c.nmat, eps, flags, s), "norm_finalize")
-        _lib.check(lib.muon_amd_normalize(mats, self.tile_prefix_ptr, c.nmat, c.ntiles, s), "normalize")
+        elts = sum(lay.numel for lay in c.layouts)
+        padded = sum(lay.mp * lay.np_ for lay in c.layouts)
+        _launch("momentum", elts * 14, lambda: _lib.check(lib.muon_amd_momentum(
+            mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
+            int(mutate_grad), s), "momentum"))
+        _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
+            mats, c.nmat, eps, flags, s), "norm_finalize"))
+        _launch("normalize", elts * 2 + padded * 4, lambda: _lib.check(lib.muon_amd_normalize(
+            mats, self.tile_prefix_ptr, c.nmat, c.ntiles, s), "normalize"))
+        flops = {
+            _plan.PH_SYRK: sum(lay.m * (lay.m + 1) * lay.n for lay in c.layouts),
+            _plan.PH_POLY: sum(lay.m * lay.m * (lay.m + 1) for lay in c.layouts),
+        }
+        f_upd = sum(2 * lay.m * lay.m * lay.n for lay in c.layouts)
         for it in range(c.steps):
-            for ph in (_plan.PH_SYRK, _plan.PH_POLY):
+            for ph, name in ((_plan.PH_SYRK, "ns_gemm/syrk"), (_plan.PH_POLY, "ns_gemm/poly")):
                 al, be, ga = c.phase_scalars(ph)
-                _lib.check(lib.muon_amd_ns_gemm(self.gemm_ptr[ph], self.sym_jobs_ptr, len(c.sym_jobs),
-                                                c.tile_class, al, be, ga, flags, s), "ns_gemm")
+                _launch(name, flops[ph], lambda ph=ph, al=al, be=be, ga=ga: _lib.check(lib.muon_amd_ns_gemm(
+                    self.gemm_ptr[ph], self.sym_jobs_ptr, len(c.sym_jobs), c.tile_class, al, be, ga,
+                    flags, s), "ns_gemm"))
             ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
             al, be, ga = c.phase_scalars(ph)
-            _lib.check(lib.muon_amd_ns_gemm(self.gemm_ptr[ph], self.full_jobs_ptr, len(c.full_jobs),
-                                            c.tile_class, al, be, ga, flags, s), "ns_gemm")
-        _lib.check(lib.muon_amd_apply(mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply")
+            _launch("ns_gemm/update", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm(
+                self.gemm_ptr[ph], self.full_jobs_ptr, len(c.full_jobs), c.tile_class, al, be, ga,
+                flags, s), "ns_gemm"))
+        _launch("apply", elts * 10, lambda: _lib.check(lib.muon_amd_apply(
+            mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply"))
 
 
 class MuonGroupEngine:
@@ -165,6 +196,6 @@ class AdamGroupEngine:
         w2 = 1 - betas[1]
         bias1 = 1 - betas[0] ** step
         bias2 = 1 - betas[1] ** step
-        _lib.check(lib.muon_amd_adam(self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels),
-                                     self.nblocks, lr, 1 - lr * weight_decay, w1, w2, eps, bias1, bias2,
-                                     _stream_ptr(self.device)), "adam")
+        _launch("adam", sum(self.numels) * 28, lambda: _lib.check(lib.muon_amd_adam(
+            self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels), self.nblocks, lr,
+            1 - lr * weight_decay, w1, w2, eps, bias1, bias2, _stream_ptr(self.device)), "adam"))

@@ -1,0 +1,207 @@
+"""Host-side logic that needs no GPU: the C ABI library loads and exports every declared symbol,
+descriptor layouts match, launch plans are well formed, and the optimizer classes keep the
+reference's constructor contract (reference muon.py:39-43, 77-79, 139-156, 206-222)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import muon_amd
+from muon_amd import _lib, plan
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ------------------------------------------------------------------------------------------
+# C ABI
+# ------------------------------------------------------------------------------------------
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "muon_amd.h")).read()
+    declared = set(re.findall(r"\b(muon_amd_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib = _lib.load()
+    assert lib.muon_amd_abi_version() == 1
+    assert lib.muon_amd_gemm_tile(0) == plan.TILE_EDGE[0] and lib.muon_amd_gemm_tile(1) == plan.TILE_EDGE[1]
+    assert lib.muon_amd_gemm_tile(7) < 0 and b"tile class" in lib.muon_amd_last_error()
+    assert lib.muon_amd_elementwise_block_elems() == plan.EW_BLOCK_ELEMS
+    assert lib.muon_amd_normalize_tile() == plan.NT_TILE
+
+
+def test_struct_layouts_match_the_library():
+    lib = _lib.load()
+    assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 112
+    assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 88
+    assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 16
+    assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 48
+
+
+def test_entry_points_reject_bad_arguments_without_a_gpu():
+    lib = _lib.load()
+    assert lib.muon_amd_ns_gemm(None, None, 1, 0, 1.0, 0.0, 0.0, 0, None) == -1
+    assert lib.muon_amd_momentum(None, None, 1, 1, 0.05, 0.95, 1, 0, None) == -1
+    assert lib.muon_amd_adam(None, None, 1, 1, 1e-3, 1.0, 0.1, 0.05, 1e-10, 0.1, 0.05, None) == -1
+    with pytest.raises(_lib.MuonAmdError):
+        _lib.check(lib.muon_amd_apply(None, None, 0, 0, 0.0, 1.0, None), "apply")
+
+
+# ------------------------------------------------------------------------------------------
+# planning
+# ------------------------------------------------------------------------------------------
+SHAPES = [(768, 3072), (3072, 768), (768, 768), (4096, 4096), (64, 216), (16384, 128), (5, 3), (1024, 4096)]
+
+
+@pytest.mark.parametrize("ref", [True, False])
+def test_plans_validate_and_cover_every_tile_once(ref):
+    lib = _lib.load()
+    chunks = plan.plan_chunks(SHAPES, 5, ref, 1 << 30)
+    seen = sorted(l.index for c in chunks for l in c.layouts)
+    assert seen == list(range(len(SHAPES)))
+    for c in chunks:
+        T = c.tile
+        assert all(plan.tile_class_for(l.m) == c.tile_class for l in c.layouts)
+        g = c.gemm_descs(1 << 20)
+        for ph in range(5):
+            jobs = c.sym_jobs if ph < 2 else c.full_jobs
+            rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class)
+            assert rc == 0, lib.muon_amd_last_error()
+        for k, l in enumerate(c.layouts):
+            mt, nt = l.mp // T, l.np_ // T
+            sj = c.sym_jobs[c.sym_jobs["desc"] == k]
+            got = sorted(zip((sj["i0"] // T).tolist(), (sj["j0"] // T).tolist()))
+            assert got == [(i, j) for i in range(mt) for j in range(i, mt)]
+            assert np.array_equal(sj["diag"], (sj["i0"] == sj["j0"]).astype(np.int32))
+            fj = c.full_jobs[c.full_jobs["desc"] == k]
+            got = sorted(zip((fj["i0"] // T).tolist(), (fj["j0"] // T).tolist()))
+            assert got == [(i, j) for i in range(mt) for j in range(nt)]
+            assert l.mp % T == 0 and l.np_ % T == 0 and l.mp >= l.m and l.np_ >= l.n
+            assert l.wide == (l.rows <= l.cols)
+        # workspace regions do not overlap and stay inside the chunk's workspace
+        regions = []
+        for l in c.layouts:
+            xb, ab = l.mp * l.np_ * 2, l.mp * l.mp * 2
+            for name in ("X", "XT0", "XT1", "A", "B", "CA"):
+                regions.append((l.off[name], l.off[name] + (xb if name.startswith("X") else ab)))
+        regions += [(c.off_partials, c.off_partials + 4 * c.nblocks), (c.off_denoms, c.off_denoms + 4 * c.nmat)]
+        regions.sort()
+        assert all(a[1] <= b[0] for a, b in zip(regions, regions[1:])) and regions[-1][1] <= c.workspace_bytes
+        assert all(r[0] % 256 == 0 for r in regions)
+        md = c.mat_descs(1 << 20)
+        md["grad"] = 4096
+        md["out"] = 8192
+        rc = lib.muon_amd_validate_mats(_lib.host_ptr(md), c.nmat, _lib.host_ptr(c.block_prefix),
+                                        _lib.host_ptr(c.tile_prefix), c.tile)
+        assert rc == 0, lib.muon_amd_last_error()
+
+
+def test_validation_catches_a_bad_table():
+    lib = _lib.load()
+    c = plan.plan_chunks([(768, 3072)], 5, True, 1 << 30)[0]
+    g = c.gemm_descs(1 << 20)
+    bad = c.full_jobs.copy()
+    bad["j0"][0] = c.layouts[0].np_          # one tile past the last column
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[2]), 1, _lib.host_ptr(bad), len(bad), c.tile_class) == -1
+    gd = g[0].copy()
+    gd["K"] = 100                            # not a multiple of the k-block
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(gd), 1, _lib.host_ptr(c.sym_jobs), len(c.sym_jobs), c.tile_class) == -1
+    low = c.sym_jobs.copy()
+    low["i0"][0], low["j0"][0] = 128, 0      # below the diagonal of a mirrored GEMM
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[0]), 1, _lib.host_ptr(low), len(low), c.tile_class) == -1
+
+
+def test_xcd_permutation_and_result_buffer():
+    for n in (1, 7, 8, 9, 136, 1000):
+        p = plan.xcd_permutation(n)
+        assert sorted(p.tolist()) == list(range(n))
+    p = plan.xcd_permutation(64)                 # block b runs on XCD b % 8: contiguous logical range per XCD
+    assert p[:8].tolist() == [0, 8, 16, 24, 32, 40, 48, 56] and p[8] == 1
+    for steps, want_tall in ((0, "XT0"), (1, "XT1"), (2, "XT0"), (5, "XT1")):
+        c = plan.ChunkPlan([(0, 300, 100), (1, 100, 300)], 0, steps, True)
+        assert c.result_buffer(c.layouts[0]) == want_tall and c.result_buffer(c.layouts[1]) == "X"
+
+
+def test_chunking_respects_the_workspace_cap():
+    shapes = [(4096, 14336)] * 6 + [(1024, 4096)] * 4 + [(768, 768)] * 3
+    one = plan.matrix_workspace_bytes(4096, 14336, 256)
+    chunks = plan.plan_chunks(shapes, 5, True, 2 * one + (1 << 20))
+    big = [c for c in chunks if any(l.n == 14336 for l in c.layouts)]
+    assert all(sum(1 for l in c.layouts if l.n == 14336) <= 2 for c in big) and len(big) >= 3
+    assert all(len({plan.tile_class_for(l.m) for l in c.layouts}) == 1 for c in chunks)
+    tiny_cap = plan.plan_chunks(shapes, 5, True, 1)           # every matrix still gets a chunk
+    assert sum(c.nmat for c in tiny_cap) == len(shapes)
+
+
+# ------------------------------------------------------------------------------------------
+# optimizer constructors (CPU tensors: construction works, stepping refuses loudly)
+# ------------------------------------------------------------------------------------------
+def test_constructor_contract_matches_the_reference():
+    a = torch.nn.Parameter(torch.zeros(4, 8))
+    b = torch.nn.Parameter(torch.zeros(16, 8))
+    c = torch.nn.Parameter(torch.zeros(8))
+    opt = muon_amd.SingleDeviceMuon([a, b])
+    assert opt.defaults == dict(lr=0.02, weight_decay=0, momentum=0.95)
+    assert [tuple(p.shape) for p in opt.param_groups[0]["params"]] == [(4, 8), (16, 8)]     # order kept
+    srt = muon_amd.Muon([a, b], lr=0.05)
+    assert [tuple(p.shape) for p in srt.param_groups[0]["params"]] == [(16, 8), (4, 8)]     # muon.py:42
+    with pytest.raises(AssertionError):
+        muon_amd.Muon((a, b))                                                             # must be a list (muon.py:41)
+    with pytest.raises(AssertionError):
+        muon_amd.Muon([])
+    groups = [dict(params=[a, b], use_muon=True), dict(params=[c], use_muon=False)]
+    aux = muon_amd.MuonWithAuxAdam(groups)
+    g0, g1 = aux.param_groups
+    assert (g0["lr"], g0["momentum"], g0["weight_decay"]) == (0.02, 0.95, 0)
+    assert (g1["lr"], g1["betas"], g1["eps"], g1["weight_decay"]) == (3e-4, (0.9, 0.95), 1e-10, 0)
+    assert [tuple(p.shape) for p in g0["params"]] == [(16, 8), (4, 8)]                      # muon.py:143
+    sd = muon_amd.SingleDeviceMuonWithAuxAdam([dict(params=[a, b], use_muon=True)])
+    assert [tuple(p.shape) for p in sd.param_groups[0]["params"]] == [(4, 8), (16, 8)]      # not sorted
+    for bad in ([dict(params=[a])], [dict(params=[a], use_muon=True, betas=(0.9, 0.9))],
+                [dict(params=[c], use_muon=False, momentum=0.9)]):
+        with pytest.raises(AssertionError):
+            muon_amd.SingleDeviceMuonWithAuxAdam(bad)
+    with pytest.raises(ValueError):
+        muon_amd.SingleDeviceMuon([a], ns_rounding="nearest")
+
+
+def test_no_cpu_fallback():
+    a = torch.nn.Parameter(torch.zeros(4, 8))
+    a.grad = torch.ones(4, 8)
+    with pytest.raises(muon_amd.MuonAmdError, match="no CPU implementation"):
+        muon_amd.SingleDeviceMuon([a]).step()
+    with pytest.raises(muon_amd.MuonAmdError):
+        muon_amd.zeropower_via_newtonschulz5(torch.ones(4, 8))
+    with pytest.raises(muon_amd.MuonAmdError):
+        muon_amd.adam_update(torch.ones(4), torch.zeros(4), torch.zeros(4), 1, (0.9, 0.95), 1e-10)
+    with pytest.raises(muon_amd.MuonAmdError):
+        muon_amd.muon_update(torch.ones(4, 8), torch.zeros(4, 8))
+    with pytest.raises(AssertionError):
+        muon_amd.zeropower_via_newtonschulz5(torch.ones(4))                                  # muon.py:275
+
+
+def test_reference_module_name_is_importable():
+    import muon
+    assert muon.MuonWithAuxAdam is muon_amd.MuonWithAuxAdam
+    assert muon.zeropower_via_newtonschulz5 is muon_amd.zeropower_via_newtonschulz5
+    import inspect
+    sig = inspect.signature(muon.muon_update)
+    assert list(sig.parameters)[:4] == ["grad", "momentum", "beta", "nesterov"]
+    assert sig.parameters["beta"].default == 0.95 and sig.parameters["nesterov"].default is True
+    assert sig.parameters["ns_steps"].default == 5
+    assert list(inspect.signature(muon.adam_update).parameters) == ["grad", "buf1", "buf2", "step", "betas", "eps"]
+    z = inspect.signature(muon.zeropower_via_newtonschulz5).parameters
+    assert z["steps"].default == 5 and z["epsilon"].default == 1e-7
+    assert plan.NS_COEFFS == (3.4445, -4.7750, 2.0315)
+
+
+def test_product_never_imports_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "muon_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)
+    assert "oracle" not in open(os.path.join(ROOT, "muon.py")).read()
