@@ -50,6 +50,8 @@ extern "C" {
  * the GEMM tile of the chunk (zero padded; zero rows/columns stay zero through the iteration).
  *   direct : rows_p x cols_p  bf16, the matrix in the orientation of the parameter
  *   transp : cols_p x rows_p  bf16, its transpose
+ * (each with its own leading dimension, which may exceed the padded width so that rows do not
+ * sit a power of two apart in memory)
  * For a wide matrix (rows <= cols) X = direct and X^T = transp; for a tall one the roles swap,
  * which is how the reference's transpose-if-tall (muon.py:278-279, 289-290) is folded into
  * indexing instead of a pass of its own.
@@ -67,6 +69,8 @@ typedef struct MuonMatDesc {
     float*    denom;       /* one float: (||u||_F + eps) as the reference forms it            */
     int32_t   rows, cols;
     int32_t   rows_p, cols_p;
+    int32_t   ld_direct;   /* leading dimension (elements) of direct and result, >= cols_p    */
+    int32_t   ld_transp;   /* leading dimension (elements) of transp, >= rows_p               */
     int32_t   src_dtype;   /* MUON_AMD_SRC_*                                                  */
     float     scale;       /* max(1, grad.size(-2)/grad.size(-1))**0.5  (muon.py:14)          */
     int32_t   part_begin;  /* first global block id of this matrix in the momentum launch     */
@@ -78,7 +82,8 @@ typedef struct MuonMatDesc {
  *     o  = bf16(t1 + t2)          -> C[i][j]  and  CT[j][i]
  *     o2 = bf16(gamma * o)        -> C2[i][j] and  C2T[j][i]
  * Any of D, C, CT, C2, C2T may be NULL.  When CT == C the job list only covers tiles with
- * j0 >= i0 and the kernel mirrors them (it skips the mirror store on diagonal tiles).
+ * their column block on or above their row block and the kernel mirrors them (tiles inside a
+ * diagonal block are stored directly and never mirrored: MuonTileJob.diag).
  * Replaces the functional roles of the reference's three Triton kernels:
  *   ns_line_1 (A = X X^T, muon.py:349-456), ns_line_2 (alpha A A^T + beta A, muon.py:464-588),
  *   ns_line_3 (a X + B X, muon.py:639-746).                                                   */
@@ -93,9 +98,9 @@ typedef struct MuonGemmDesc {
 /* One output tile of one matrix. */
 typedef struct MuonTileJob {
     int32_t desc;   /* index into the MuonGemmDesc table of the launch */
-    int32_t i0;     /* first output row  (multiple of the tile)        */
-    int32_t j0;     /* first output col  (multiple of the tile)        */
-    int32_t diag;   /* 1 when i0 == j0 of a mirrored (symmetric) GEMM  */
+    int32_t i0;     /* first output row  (multiple of the tile rows)   */
+    int32_t j0;     /* first output col  (multiple of the tile cols)   */
+    int32_t diag;   /* 1 when a mirrored (symmetric) GEMM's tile lies in a diagonal block */
 } MuonTileJob;
 
 /* One tensor of the auxiliary Adam group. */
@@ -122,9 +127,12 @@ size_t muon_amd_sizeof_adam_desc(void);
 int muon_amd_elementwise_block_elems(void);
 int muon_amd_normalize_tile(void);
 
-/* GEMM tile classes.  tile_class 0: 128x128 output tile, 256 threads; 1: 256x256, 512 threads.
- * Returns the tile edge, or a negative code for an unknown class. */
-int muon_amd_gemm_tile(int tile_class);
+/* GEMM tile classes (rows x cols of the output tile a workgroup computes):
+ *   0: 128 x 128 (4 waves, two workgroups per CU)   1: 256 x 256 (8 waves, one workgroup per CU)
+ * Padded matrix sizes must be multiples of the larger of the two.  Return the tile extent, or
+ * a negative code for an unknown class. */
+int muon_amd_gemm_tile_rows(int tile_class);
+int muon_amd_gemm_tile_cols(int tile_class);
 
 /* ---- host-side validation (no GPU work): checks host copies of the tables a launch will
  *      use against what the kernels assume.  Call before uploading them.                 ---- */

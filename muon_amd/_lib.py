@@ -25,7 +25,7 @@ MAT_DESC = np.dtype(
     [("grad", "<u8"), ("momentum", "<u8"), ("param", "<u8"), ("out", "<u8"), ("u", "<u8"),
      ("direct", "<u8"), ("transp", "<u8"), ("result", "<u8"), ("partials", "<u8"),
      ("denom", "<u8"), ("rows", "<i4"), ("cols", "<i4"), ("rows_p", "<i4"), ("cols_p", "<i4"),
-     ("src_dtype", "<i4"), ("scale", "<f4"), ("part_begin", "<i4"), ("part_end", "<i4")],
+     ("ld_direct", "<i4"), ("ld_transp", "<i4"), ("src_dtype", "<i4"), ("scale", "<f4"), ("part_begin", "<i4"), ("part_end", "<i4")],
     align=True)
 GEMM_DESC = np.dtype(
     [("P", "<u8"), ("Q", "<u8"), ("D", "<u8"), ("C", "<u8"), ("CT", "<u8"), ("C2", "<u8"),
@@ -52,7 +52,8 @@ SIGNATURES = {
     "muon_amd_sizeof_adam_desc": (ctypes.c_size_t, []),
     "muon_amd_elementwise_block_elems": (_c_int, []),
     "muon_amd_normalize_tile": (_c_int, []),
-    "muon_amd_gemm_tile": (_c_int, [_c_int]),
+    "muon_amd_gemm_tile_rows": (_c_int, [_c_int]),
+    "muon_amd_gemm_tile_cols": (_c_int, [_c_int]),
     "muon_amd_validate_gemm": (_c_int, [_vp, _c_int, _vp, _c_int, _c_int]),
     "muon_amd_validate_mats": (_c_int, [_vp, _c_int, _vp, _vp, _c_int]),
     "muon_amd_momentum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _vp]),

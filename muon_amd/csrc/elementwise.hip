@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
         o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
         o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
         o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
-        *reinterpret_cast<uint4*>(d.direct + static_cast<int64_t>(gr) * d.cols_p + gc) = o;
+        *reinterpret_cast<uint4*>(d.direct + static_cast<int64_t>(gr) * d.ld_direct + gc) = o;
 #pragma unroll
         for (int k = 0; k < 8; ++k) tile[r][cc + k] = v[k];
     }
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
         o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
         o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
         o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
-        *reinterpret_cast<uint4*>(d.transp + static_cast<int64_t>(C0 + tr) * d.rows_p + R0 + tc) = o;
+        *reinterpret_cast<uint4*>(d.transp + static_cast<int64_t>(C0 + tr) * d.ld_transp + R0 + tc) = o;
     }
 }
 
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
         for (int it = 0; it < EW_ITERS; ++it) {
             const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
             const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
-            ov[it] = *reinterpret_cast<const uint2*>(res + static_cast<int64_t>(rr) * d.cols_p + cc);
+            ov[it] = *reinterpret_cast<const uint2*>(res + static_cast<int64_t>(rr) * d.ld_direct + cc);
             pv[it] = p ? *reinterpret_cast<const float4*>(p + e) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
                 const int64_t e = e0 + k;
                 if (e >= numel) break;
                 const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
-                const float us = round_bf(bf2f(res[static_cast<int64_t>(rr) * d.cols_p + cc]) * scale);
+                const float us = round_bf(bf2f(res[static_cast<int64_t>(rr) * d.ld_direct + cc]) * scale);
                 if (p) p[e] = fmaf(neg_lr, us, p[e] * wd_factor);
                 if (out) out[e] = f2bf(us);
             }
@@ -368,6 +368,10 @@ int muon_amd_validate_mats(const MuonMatDesc* descs, int nmat, const int32_t* bl
                          d.cols_p % tile_edge == 0,
                      "mat %d: padded %dx%d does not cover %dx%d in tiles of %d", i, d.rows_p,
                      d.cols_p, d.rows, d.cols, tile_edge);
+        MUON_REQUIRE(d.ld_direct >= d.cols_p && d.ld_transp >= d.rows_p && d.ld_direct % 8 == 0 &&
+                         d.ld_transp % 8 == 0,
+                     "mat %d: leading dimensions %d/%d for padded %dx%d", i, d.ld_direct, d.ld_transp,
+                     d.rows_p, d.cols_p);
         MUON_REQUIRE(d.grad && d.u && d.direct && d.transp && d.result && d.partials && d.denom,
                      "mat %d: null workspace or source pointer", i);
         MUON_REQUIRE(d.param || d.out, "mat %d: neither param nor out given", i);

@@ -11,74 +11,299 @@
 // mirror half of a symmetric result, or X^T for the next iteration), and optionally a scaled
 // copy (c*A).  Symmetric results only compute tiles on or above the diagonal.
 //
-// A launch covers a job list of output tiles drawn from many matrices.  A workgroup computes
-// one BM x BN tile with BK = 64: global -> registers -> LDS (double buffered, rows padded by
-// 16 bytes so the ds_read_b128 fragment loads are bank-conflict free), then
-// v_mfma_f32_32x32x16_bf16 with fp32 accumulation.
+// A launch covers a job list of output tiles drawn from many matrices; a workgroup computes one
+// BM x BN tile:
+//   * global_load_lds_dwordx4 streams the operand tiles straight into an LDS ring (no register
+//     staging) in k-blocks of BK = 64, so every request is a full 128-byte line of one operand
+//     row; the ring keeps a block and a half in flight while the current one is multiplied;
+//   * LDS rows are 128 bytes (8 chunks of 16 bytes); chunk c of row r sits at position
+//     c ^ ((r >> 1) & 7), so the 1 KiB-contiguous DMA writes and the ds_read_b128 fragment reads
+//     are both bank-conflict free;
+//   * each wave owns a 128 x 64 (or 64 x 64) sub-tile as 32 x 32 v_mfma_f32_32x32x16_bf16 tiles
+//     with fp32 accumulation;
+//   * the epilogue moves tiles between the "lane owns a column" accumulator layout and the
+//     "lane owns a row" layout with two MFMAs against a permuted identity, so that the addend is
+//     read and both output orientations are written with wide, coalesced accesses staged through
+//     wave-private LDS.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace muon_amd {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-// 16-byte load through the global (not flat) address space: pointers fetched from a descriptor
-// are generic to the compiler, and a flat load would also count against the LDS wait counter.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ u32x4 gload16(const uint16_t* p) {
-    return *(const __attribute__((address_space(1))) u32x4*)(p);
+
+// Accesses through the global (not flat) address space: pointers fetched from a descriptor are
+// generic to the compiler, and a flat access would also count against the LDS wait counter.
+__device__ __forceinline__ u32x2 gload8(const uint16_t* p) {
+    return *(const __attribute__((address_space(1))) u32x2*)(p);
 }
-__device__ __forceinline__ uint16_t gload2(const uint16_t* p) {
-    return *(const __attribute__((address_space(1))) uint16_t*)(p);
-}
-__device__ __forceinline__ void gstore2(uint16_t* p, uint16_t v) {
-    *(__attribute__((address_space(1))) uint16_t*)(p) = v;
-}
-__device__ __forceinline__ void gstore8(uint16_t* p, u32x2 v) {
-    *(__attribute__((address_space(1))) u32x2*)(p) = v;
+__device__ __forceinline__ void gstore16(uint16_t* p, u32x4 v) {
+    *(__attribute__((address_space(1))) u32x4*)(p) = v;
 }
 
-constexpr int BK = 64;           // k extent of one LDS stage
-constexpr int LDK = BK + 8;      // padded LDS row length in elements (144 bytes)
+constexpr int BK = 64;   // k extent of one ring stage (128 bytes per LDS row)
+constexpr int ROW_BYTES = BK * 2;
 
-template <int BM, int BN, int WGM, int WGN>
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS at
+// lds_addr + lane*16 (lds_addr wave-uniform).  Issued through inline assembly so that the
+// compiler's wait-count insertion does not serialise the ring; completion is awaited explicitly
+// with s_waitcnt vmcnt(n) before the workgroup barrier that publishes a stage.
+__device__ __forceinline__ void dma16(const uint16_t* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n"
+                 :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained); n < 16.
+#define NS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | (n))
+
+// ---------------------------------------------------------------------------------------------
+// Epilogue helpers
+// ---------------------------------------------------------------------------------------------
+// out = V^T for a 32 x 32 tile of bf16-representable values held in accumulator layout (lane =
+// column l%32, register 4q+e = row 8q + 4(l/32) + e).  V goes in as the A operand; id0/id1 are the
+// B operands with B[slot][j] = (row(slot) == j), where slot (g, t) of k-block h carries tile row
+// 16h + 8(t/4) + 4g + t%4 -- exactly the rows registers 8h .. 8h+7 hold.  bf16 x 1.0 products and
+// sums of a single non-zero term are exact in the fp32 accumulator.
+__device__ __forceinline__ f32x16 tile_transpose_bf16(const float (&v)[16], bf16x8 id0, bf16x8 id1) {
+    bf16x8 f0, f1;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        f0[t] = static_cast<__bf16>(v[t]);
+        f1[t] = static_cast<__bf16>(v[8 + t]);
+    }
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f0, id0, z, 0, 0, 0);
+    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f1, id1, z, 0, 0, 0);
+    return z;
+}
+
+// bf16(gamma * x) for 8 packed bf16 values.
+__device__ __forceinline__ u32x4 scale_bf16x8(u32x4 v, float gamma) {
+    u32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float lo = gamma * __uint_as_float(v[k] << 16);
+        const float hi = gamma * __uint_as_float(v[k] & 0xffff0000u);
+        r[k] = pack2bf(lo, hi);
+    }
+    return r;
+}
+
+// Wave-private staging bytes the epilogue needs for a WM x WN wave tile (rows padded by 16 B).
+constexpr int epilogue_stage_bytes(int WM, int WN) {
+    return (WM * (WN * 2 + 16) > WN * (WM * 2 + 16)) ? WM * (WN * 2 + 16) : WN * (WM * 2 + 16);
+}
+
+// Per 32 x 32 tile: t1 = alpha*acc -> row-owning layout -> + beta*D (8-byte loads) -> o (bf16)
+// -> staged row-major in LDS -> 16-byte coalesced stores of C (and gamma*o to C2); o moved back
+// to the column-owning layout -> staged -> 16-byte coalesced stores of CT (and C2T).
+template <bool HAS_D, int WGN, int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const MuonGemmDesc& d,
+                                                 const MuonTileJob& job, float alpha, float beta,
+                                                 float gamma, bool round_terms, char* stage) {
+    constexpr int DROW = WN * 2 + 16;   // staged row pitch in bytes, direct orientation
+    constexpr int TROW = WM * 2 + 16;   // transposed orientation
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lr = lane & 31, g = lane >> 5;
+    const int row0 = job.i0 + wm * WM, col0 = job.j0 + wn * WN;   // origin of this wave's sub-tile
+    const bool do_d = d.C != nullptr;
+    const bool do_t = d.CT != nullptr && !(job.diag && d.CT == d.C);
+
+    bf16x8 id0, id1;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const int rho = 8 * (t >> 2) + 4 * g + (t & 3);
+        id0[t] = static_cast<__bf16>(rho == lr ? 1.0f : 0.0f);
+        id1[t] = static_cast<__bf16>(16 + rho == lr ? 1.0f : 0.0f);
+    }
+
+    // addend: lane owns row (a*32 + lr) and columns b*32 + 8q + 4g .. +4 -> one 8-byte load each,
+    // all issued before the first is used.  D may alias C (in-place a*X + B*X): every load of
+    // this wave's sub-tile precedes its stores through the data dependence on o.
+    u32x2 dv[TM][TN][4];
+    if (HAS_D) {
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    dv[a][b][q] = gload8(d.D + static_cast<size_t>(row0 + a * 32 + lr) * d.ldd + col0 +
+                                         b * 32 + 8 * q + 4 * g);
+    }
+
+    uint32_t ot[TM][TN][8];   // results moved back to accumulator layout, packed bf16 pairs
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+#pragma unroll
+        for (int b = 0; b < TN; ++b) {
+            f32x16 u;
+            if (round_terms) {
+                float t1[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) t1[i] = round_bf(alpha * acc[a][b][i]);
+                u = tile_transpose_bf16(t1, id0, id1);
+            } else {
+                // keep ~16 mantissa bits: transpose a bf16 head and a bf16 tail and add them
+                float hi[16], lo[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float v = alpha * acc[a][b][i];
+                    hi[i] = round_bf(v);
+                    lo[i] = round_bf(v - hi[i]);
+                }
+                const f32x16 uh = tile_transpose_bf16(hi, id0, id1);
+                const f32x16 ul = tile_transpose_bf16(lo, id0, id1);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) u[i] = uh[i] + ul[i];
+            }
+            float o[16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float dd[4] = {0.f, 0.f, 0.f, 0.f};
+                if (HAS_D) {
+                    dd[0] = __uint_as_float(dv[a][b][q].x << 16);
+                    dd[1] = __uint_as_float(dv[a][b][q].x & 0xffff0000u);
+                    dd[2] = __uint_as_float(dv[a][b][q].y << 16);
+                    dd[3] = __uint_as_float(dv[a][b][q].y & 0xffff0000u);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float t2 = HAS_D ? beta * dd[e] : 0.f;
+                    if (round_terms) t2 = round_bf(t2);
+                    o[4 * q + e] = round_bf(u[4 * q + e] + t2);
+                }
+                if (do_d) {
+                    u32x2 pk;
+                    pk.x = pack2bf(o[4 * q], o[4 * q + 1]);
+                    pk.y = pack2bf(o[4 * q + 2], o[4 * q + 3]);
+                    *reinterpret_cast<u32x2*>(stage + (a * 32 + lr) * DROW + (b * 32 + 8 * q + 4 * g) * 2) = pk;
+                }
+            }
+            if (do_t) {
+                const f32x16 w = tile_transpose_bf16(o, id0, id1);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) ot[a][b][k] = pack2bf(w[2 * k], w[2 * k + 1]);
+            }
+        }
+    }
+
+    if (do_d) {
+        constexpr int CPR = WN / 8, RPI = 64 / CPR;     // 16-byte chunks per row, rows per wave store
+        const int r = lane / CPR, ch = lane % CPR;
+#pragma unroll
+        for (int it = 0; it < WM / RPI; ++it) {
+            const int row = it * RPI + r;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
+            const size_t off = static_cast<size_t>(row0 + row) * d.ldc + col0 + ch * 8;
+            gstore16(d.C + off, v);
+            if (d.C2) gstore16(d.C2 + off, scale_bf16x8(v, gamma));
+        }
+    }
+    if (do_t) {
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    u32x2 pk;
+                    pk.x = ot[a][b][2 * q];
+                    pk.y = ot[a][b][2 * q + 1];
+                    *reinterpret_cast<u32x2*>(stage + (b * 32 + lr) * TROW + (a * 32 + 8 * q + 4 * g) * 2) = pk;
+                }
+        constexpr int CPR = WM / 8, RPI = 64 / CPR;
+        const int r = lane / CPR, ch = lane % CPR;
+#pragma unroll
+        for (int it = 0; it < WN / RPI; ++it) {
+            const int row = it * RPI + r;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
+            const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + ch * 8;
+            gstore16(d.CT + off, v);
+            if (d.C2T) gstore16(d.C2T + off, scale_bf16x8(v, gamma));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The kernel
+// ---------------------------------------------------------------------------------------------
+// The LDS ring holds NHALF = 5 half-stages; a half-stage is the P rows or the Q rows of one
+// k-block (BT rows x 128 bytes).  Half-stages are issued in the order P0 Q0 P1 Q1 P2 ...; block kb
+// needs halves 2kb and 2kb+1.  While block kb is multiplied, half 2kb+2 (issued one iteration
+// earlier) and halves 2kb+3, 2kb+4 (issued at the top of this iteration into the two slots
+// block kb-1 vacated) are in flight, so the load pipe always has a queued request and every
+// request is a full 128-byte line.
+constexpr int NHALF = 5;
+
+template <int BT_, int WGM_, int WGN_, int MINB_>
 struct GemmCfg {
-    static constexpr int NT = WGM * WGN * 64;
-    static constexpr int WM = BM / WGM, WN = BN / WGN;
-    static constexpr int TM = WM / 32, TN = WN / 32;
-    static constexpr int ROWS_PER_PASS = NT / 8;          // 8 x 16-byte chunks per 64-wide row
-    static constexpr int PCH = BM / ROWS_PER_PASS, QCH = BN / ROWS_PER_PASS;
-    static constexpr int STAGE = (BM + BN) * LDK;         // elements per LDS stage
-    static constexpr size_t LDS_BYTES = 2u * STAGE * sizeof(uint16_t);
-    static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tile must be MFMA tiles");
-    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "loader must tile the stage");
+    static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_;
+    static constexpr int NW = WGM * WGN, NT = NW * 64;
+    static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    static constexpr int HALF_BYTES = BT_ * ROW_BYTES;
+    static constexpr int DPH = BT_ / 8 / NW;          // DMA instructions (8 rows each) per wave per half
+    static constexpr size_t RING_BYTES = static_cast<size_t>(NHALF) * HALF_BYTES;
+    static constexpr size_t EPI_BYTES = static_cast<size_t>(NW) * epilogue_stage_bytes(WM, WN);
+    static constexpr size_t LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
+    static_assert(BT_ % (8 * NW) == 0, "DMA tiling");
+    static_assert(3 * DPH < 16, "vmcnt immediate");
+    static_assert(NW % 2 == 0, "swizzle parity assumes an even wave count");
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be MFMA tiles");
+    static_assert(LDS_BYTES <= 163840, "LDS capacity of a gfx950 CU");
 };
 
-template <int BM, int BN, int WGM, int WGN, int MINB>
-__global__ __launch_bounds__(WGM * WGN * 64, MINB) void ns_gemm_kernel(
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, float alpha,
-    float beta, float gamma, int round_terms) {
-    using Cfg = GemmCfg<BM, BN, WGM, WGN>;
-    constexpr int NT = Cfg::NT, TM = Cfg::TM, TN = Cfg::TN, PCH = Cfg::PCH, QCH = Cfg::QCH;
+    float beta, float gamma, int flags) {
+    constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
+    constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
     extern __shared__ __align__(16) uint16_t lds[];
-
     const MuonTileJob job = jobs[blockIdx.x];
     const MuonGemmDesc d = descs[job.desc];
     const int i0 = job.i0, j0 = job.j0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
 
-    // ---- global -> register -> LDS staging --------------------------------------------------
-    const int crow = tid >> 3, cchunk = (tid & 7) * 8;
-    const uint16_t* __restrict__ Pg = d.P + static_cast<size_t>(i0 + crow) * d.ldp + cchunk;
-    const uint16_t* __restrict__ Qg = d.Q + static_cast<size_t>(j0 + crow) * d.ldq + cchunk;
-    const size_t pstep = static_cast<size_t>(Cfg::ROWS_PER_PASS) * d.ldp;
-    const size_t qstep = static_cast<size_t>(Cfg::ROWS_PER_PASS) * d.ldq;
-    uint16_t* const lds_p = lds + crow * LDK + cchunk;
-    uint16_t* const lds_q = lds + (BM + crow) * LDK + cchunk;
+    // ---- DMA addressing: instruction j of this wave fills half-stage rows (j*NW + wave)*8 .. +8;
+    //      lane -> row + lane/8, LDS chunk position lane%8, i.e. global chunk (lane%8) ^ swizzle,
+    //      swizzle = (row >> 1) & 7 = 4*(wave & 1) + lane/16 ---------------------------------------
+    const int gchunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
+    const uint16_t* srcp[DPH];
+    const uint16_t* srcq[DPH];
+#pragma unroll
+    for (int j = 0; j < DPH; ++j) {
+        const int r = (j * NW + wave) * 8 + (lane >> 3);
+        srcp[j] = d.P + static_cast<size_t>(i0 + r) * d.ldp + gchunk * 8;
+        srcq[j] = d.Q + static_cast<size_t>(j0 + r) * d.ldq + gchunk * 8;
+    }
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint16_t*)lds));
+    const uint32_t dst0 = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
 
-    u32x4 pr[PCH], qr[QCH];
+    // half h = 2*kb (+1): P (Q) rows of k-block kb, into ring slot h % NHALF
+#define NS_ISSUE_HALF(src_, kb_, slot_)                                                        \
+    do {                                                                                       \
+        _Pragma("unroll") for (int j_ = 0; j_ < DPH; ++j_)                                     \
+            dma16(src_[j_] + static_cast<size_t>(kb_) * BK,                                    \
+                  dst0 + (slot_) * HALF_BYTES + j_ * NW * 1024);                               \
+    } while (0)
+
+    // ---- fragment addressing (bytes): lane l reads row l%32, chunk 2*ks + l/32 -------------
+    const int swz = (lane >> 1) & 7;
+    const int c0 = (lane >> 5) ^ swz;
+    const char* const ldsb = reinterpret_cast<const char*>(lds);
+    const char* const pfrag = ldsb + (wm * WM + (lane & 31)) * ROW_BYTES;
+    const char* const qfrag = ldsb + (wn * WN + (lane & 31)) * ROW_BYTES;
+    const int koff[4] = {c0 * 16, (c0 ^ 2) * 16, (c0 ^ 4) * 16, (c0 ^ 6) * 16};
+
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int a = 0; a < TM; ++a)
@@ -87,126 +312,128 @@ __global__ __launch_bounds__(WGM * WGN * 64, MINB) void ns_gemm_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-    // fragment read offsets: lane l reads row (l % 32), k offset (l / 32) * 8 of each 32 x 16 slab
-    const int frag_off = (lane & 31) * LDK + (lane >> 5) * 8;
-    const uint16_t* const lds_pw = lds + (wm * Cfg::WM) * LDK + frag_off;
-    const uint16_t* const lds_qw = lds + (BM + wn * Cfg::WN) * LDK + frag_off;
-
-#define NS_GLOAD(kb_)                                                                       \
-    do {                                                                                    \
-        _Pragma("unroll") for (int i_ = 0; i_ < PCH; ++i_) pr[i_] =                         \
-            gload16(Pg + i_ * pstep + static_cast<size_t>(kb_) * BK);                       \
-        _Pragma("unroll") for (int i_ = 0; i_ < QCH; ++i_) qr[i_] =                         \
-            gload16(Qg + i_ * qstep + static_cast<size_t>(kb_) * BK);                       \
-    } while (0)
-#define NS_LSTORE(stage_)                                                                   \
-    do {                                                                                    \
-        _Pragma("unroll") for (int i_ = 0; i_ < PCH; ++i_) *reinterpret_cast<u32x4*>(       \
-            lds_p + (stage_) * Cfg::STAGE + i_ * Cfg::ROWS_PER_PASS * LDK) = pr[i_];        \
-        _Pragma("unroll") for (int i_ = 0; i_ < QCH; ++i_) *reinterpret_cast<u32x4*>(       \
-            lds_q + (stage_) * Cfg::STAGE + i_ * Cfg::ROWS_PER_PASS * LDK) = qr[i_];        \
-    } while (0)
-#define NS_COMPUTE(stage_)                                                                  \
-    do {                                                                                    \
-        const uint16_t* ps_ = lds_pw + (stage_) * Cfg::STAGE;                               \
-        const uint16_t* qs_ = lds_qw + (stage_) * Cfg::STAGE;                               \
-        _Pragma("unroll") for (int ks_ = 0; ks_ < BK / 16; ++ks_) {                         \
-            bf16x8 af_[TM], bf_[TN];                                                        \
-            _Pragma("unroll") for (int a_ = 0; a_ < TM; ++a_) af_[a_] =                     \
-                *reinterpret_cast<const bf16x8*>(ps_ + a_ * 32 * LDK + ks_ * 16);           \
-            _Pragma("unroll") for (int b_ = 0; b_ < TN; ++b_) bf_[b_] =                     \
-                *reinterpret_cast<const bf16x8*>(qs_ + b_ * 32 * LDK + ks_ * 16);           \
-            _Pragma("unroll") for (int a_ = 0; a_ < TM; ++a_)                               \
-                _Pragma("unroll") for (int b_ = 0; b_ < TN; ++b_) acc[a_][b_] =             \
-                    __builtin_amdgcn_mfma_f32_32x32x16_bf16(af_[a_], bf_[b_], acc[a_][b_],  \
-                                                            0, 0, 0);                       \
-        }                                                                                   \
-    } while (0)
-
     const int nk = d.K / BK;
-    NS_GLOAD(0);
-    NS_LSTORE(0);
-    __syncthreads();
-    int cur = 0;
-    for (int kb = 1; kb < nk; ++kb) {
-        NS_GLOAD(kb);              // next k-block: in flight while the current one is multiplied
-        __builtin_amdgcn_sched_barrier(0);   // keep the loads ahead of the MFMA block
-        NS_COMPUTE(cur);
-        __builtin_amdgcn_sched_barrier(0);
-        NS_LSTORE(cur ^ 1);
-        __syncthreads();
-        cur ^= 1;
+    // prologue: halves 0..4 = P0 Q0 P1 Q1 P2
+    NS_ISSUE_HALF(srcp, 0, 0);
+    NS_ISSUE_HALF(srcq, 0, 1);
+    if (nk > 1) {
+        NS_ISSUE_HALF(srcp, 1, 2);
+        NS_ISSUE_HALF(srcq, 1, 3);
     }
-    NS_COMPUTE(cur);
-#undef NS_GLOAD
-#undef NS_LSTORE
-#undef NS_COMPUTE
+    if (nk > 2) NS_ISSUE_HALF(srcp, 2, 4);
 
-    // ---- epilogue ------------------------------------------------------------------------------
-    // acc[a][b][i] is output (row, col) = (rb + 8*(i/4) + (i%4), cb) with
-    //   rb = i0 + wm*WM + a*32 + 4*(lane/32),  cb = j0 + wn*WN + b*32 + lane%32.
-    const bool mirror_ok = !(job.diag && d.CT == d.C);
-    const uint16_t* D = d.D;   // may alias C (in-place a*X + B*X): no restrict
+    int sp = 0, sq = 1;                 // ring slots of the P and Q halves of block kb
+    for (int kb = 0; kb < nk; ++kb) {
+        // halves 2kb and 2kb+1 have landed once only the younger halves are pending
+        if (kb == 0) {
+            if (nk > 2) NS_WAIT_VMCNT(3 * DPH);
+            else if (nk > 1) NS_WAIT_VMCNT(2 * DPH);
+            else NS_WAIT_VMCNT(0);
+        } else {
+            if (kb + 1 < nk) NS_WAIT_VMCNT(DPH);
+            else NS_WAIT_VMCNT(0);
+        }
+        __syncthreads();   // block kb visible to all waves; the two slots of block kb-1 are free
+        // halves 2kb+3 = Q(kb+1) and 2kb+4 = P(kb+2) go into the slots of halves 2kb-2, 2kb-1.
+        // Their 2*DPH DMA instructions are spread over the k-steps below, between the MFMAs: a
+        // burst right after the barrier would hold every wave in the memory-issue queue while
+        // the matrix pipe sits idle.
+        int s3 = sq + 2; s3 = s3 >= NHALF ? s3 - NHALF : s3;     // (2kb+3) % 5
+        int s4 = sp + 4; s4 = s4 >= NHALF ? s4 - NHALF : s4;     // (2kb+4) % 5
+        const bool issue_q = kb >= 1 && kb + 1 < nk;
+        const bool issue_p = kb >= 1 && kb + 2 < nk;
+        const uint16_t* const* dsrc[2] = {srcq, srcp};
+        const uint32_t ddst[2] = {dst0 + s3 * HALF_BYTES, dst0 + s4 * HALF_BYTES};
+        const size_t dk[2] = {static_cast<size_t>(kb + 1) * BK, static_cast<size_t>(kb + 2) * BK};
+        const bool dgo[2] = {issue_q, issue_p};
+        constexpr int KSTEPS = BK / 16;
+        constexpr int DPK = 2 * DPH / KSTEPS;                    // DMA instructions per k-step
+        static_assert(2 * DPH % KSTEPS == 0 && DPH % DPK == 0, "DMA instructions must spread evenly");
+
+        const char* const pf = pfrag + sp * HALF_BYTES;
+        const char* const qf = qfrag + sq * HALF_BYTES;
+        // fragments are double buffered: the ds_reads of k-step ks+1 are issued ahead of the
+        // MFMAs of k-step ks, so the matrix pipe never waits for LDS latency inside a block
+        bf16x8 af[2][TM], bfr[2][TN];
 #pragma unroll
-    for (int a = 0; a < TM; ++a) {
+        for (int a = 0; a < TM; ++a)
+            af[0][a] = *reinterpret_cast<const bf16x8*>(pf + a * 32 * ROW_BYTES + koff[0]);
 #pragma unroll
-        for (int b = 0; b < TN; ++b) {
-            const int cb = j0 + wn * Cfg::WN + b * 32 + (lane & 31);
+        for (int b = 0; b < TN; ++b)
+            bfr[0][b] = *reinterpret_cast<const bf16x8*>(qf + b * 32 * ROW_BYTES + koff[0]);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int rb = i0 + wm * Cfg::WM + a * 32 + 8 * q + 4 * (lane >> 5);
-                float o[4], o2[4];
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const int cur = ks & 1, nxt = cur ^ 1;
+            if (ks + 1 < KSTEPS) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float t1 = alpha * acc[a][b][4 * q + e];
-                    float t2 = 0.f;
-                    if (D) t2 = beta * bf2f(gload2(D + static_cast<size_t>(rb + e) * d.ldd + cb));
-                    if (round_terms) {
-                        t1 = round_bf(t1);
-                        t2 = round_bf(t2);
-                    }
-                    o[e] = round_bf(t1 + t2);
-                    o2[e] = gamma * o[e];
-                }
-                if (d.C) {
+                for (int a = 0; a < TM; ++a)
+                    af[nxt][a] = *reinterpret_cast<const bf16x8*>(pf + a * 32 * ROW_BYTES + koff[ks + 1]);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        gstore2(d.C + static_cast<size_t>(rb + e) * d.ldc + cb, f2bf(o[e]));
-                }
-                if (d.C2) {
+                for (int b = 0; b < TN; ++b)
+                    bfr[nxt][b] = *reinterpret_cast<const bf16x8*>(qf + b * 32 * ROW_BYTES + koff[ks + 1]);
+                __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
+            }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        gstore2(d.C2 + static_cast<size_t>(rb + e) * d.ldc + cb, f2bf(o2[e]));
-                }
-                if (mirror_ok) {
-                    if (d.CT) {
-                        u32x2 pk;
-                        pk.x = pack2bf(o[0], o[1]);
-                        pk.y = pack2bf(o[2], o[3]);
-                        gstore8(d.CT + static_cast<size_t>(cb) * d.ldct + rb, pk);
-                    }
-                    if (d.C2T) {
-                        u32x2 pk;
-                        pk.x = pack2bf(o2[0], o2[1]);
-                        pk.y = pack2bf(o2[2], o2[3]);
-                        gstore8(d.C2T + static_cast<size_t>(cb) * d.ldct + rb, pk);
-                    }
+            for (int a = 0; a < TM; ++a) {
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][a], bfr[cur][b], acc[a][b], 0, 0, 0);
+                // one DMA instruction after each of the first DPK rows of MFMAs of this k-step
+                if (a < DPK) {
+                    const int jj = ks * DPK + a;                 // 0 .. 2*DPH-1, Q half first
+                    const int h = jj / DPH, j = jj % DPH;
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        sp += 2; sp = sp >= NHALF ? sp - NHALF : sp;
+        sq += 2; sq = sq >= NHALF ? sq - NHALF : sq;
     }
+#undef NS_ISSUE_HALF
+    __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
+    char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
+    const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
+    if (d.D) ns_epilogue_impl<true, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
+    else ns_epilogue_impl<false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
 }
 
+// Tile classes: square output tile, waves, workgroups per CU.
+//   0: 128 x 128, 4 waves of 64 x 64, two workgroups per CU   (short side below 1024)
+//   1: 256 x 256, 8 waves of 128 x 64, one workgroup per CU   (large matrices)
+typedef GemmCfg<128, 2, 2, 2> Cfg0;
+typedef GemmCfg<256, 2, 4, 1> Cfg1;
+constexpr int kNumTileClasses = 2;
+
 struct TileClass {
-    int edge;
-    int threads;
+    int bm, bn, threads;
     size_t lds_bytes;
 };
-
-static const TileClass kTileClasses[2] = {
-    {128, GemmCfg<128, 128, 2, 2>::NT, GemmCfg<128, 128, 2, 2>::LDS_BYTES},
-    {256, GemmCfg<256, 256, 2, 4>::NT, GemmCfg<256, 256, 2, 4>::LDS_BYTES},
+static const TileClass kTileClasses[kNumTileClasses] = {
+    {Cfg0::BM, Cfg0::BN, Cfg0::NT, Cfg0::LDS_BYTES},
+    {Cfg1::BM, Cfg1::BN, Cfg1::NT, Cfg1::LDS_BYTES},
 };
+
+template <typename Cfg>
+static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
+                       float beta, float gamma, int flags, hipStream_t s) {
+    static bool attr_set = false;
+    auto kern = ns_gemm_kernel<Cfg>;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
+            set_error("ns_gemm: cannot raise dynamic LDS to %zu bytes", Cfg::LDS_BYTES);
+            return MUON_AMD_ELAUNCH;
+        }
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs, alpha, beta,
+                       gamma, flags);
+    return check_launch("ns_gemm");
+}
 
 }  // namespace muon_amd
 
@@ -214,32 +441,39 @@ using namespace muon_amd;
 
 extern "C" {
 
-int muon_amd_gemm_tile(int tile_class) {
-    MUON_REQUIRE(tile_class == 0 || tile_class == 1, "gemm_tile: unknown tile class %d", tile_class);
-    return kTileClasses[tile_class].edge;
+int muon_amd_gemm_tile_rows(int tile_class) {
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "gemm_tile_rows: unknown tile class %d", tile_class);
+    return kTileClasses[tile_class].bm;
+}
+
+int muon_amd_gemm_tile_cols(int tile_class) {
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "gemm_tile_cols: unknown tile class %d", tile_class);
+    return kTileClasses[tile_class].bn;
 }
 
 int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJob* jobs,
                            int njobs, int tile_class) {
     MUON_REQUIRE(descs && jobs, "validate_gemm: null table");
-    MUON_REQUIRE(tile_class == 0 || tile_class == 1, "validate_gemm: unknown tile class %d", tile_class);
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "validate_gemm: unknown tile class %d", tile_class);
     MUON_REQUIRE(ndesc > 0 && njobs > 0, "validate_gemm: ndesc=%d njobs=%d", ndesc, njobs);
-    const int T = kTileClasses[tile_class].edge;
+    const int TR = kTileClasses[tile_class].bm, TC = kTileClasses[tile_class].bn;
     for (int i = 0; i < ndesc; ++i) {
         const MuonGemmDesc& d = descs[i];
         MUON_REQUIRE(d.P && d.Q, "gemm desc %d: null operand", i);
         MUON_REQUIRE(d.C || d.CT, "gemm desc %d: no output", i);
         MUON_REQUIRE(d.K > 0 && d.K % BK == 0, "gemm desc %d: K=%d is not a positive multiple of %d", i, d.K, BK);
-        MUON_REQUIRE(d.rows > 0 && d.colsn > 0 && d.rows % T == 0 && d.colsn % T == 0,
-                     "gemm desc %d: output %dx%d is not in tiles of %d", i, d.rows, d.colsn, T);
+        MUON_REQUIRE(d.rows > 0 && d.colsn > 0 && d.rows % TR == 0 && d.colsn % TC == 0,
+                     "gemm desc %d: output %dx%d is not in tiles of %dx%d", i, d.rows, d.colsn, TR, TC);
         MUON_REQUIRE(d.ldp >= d.K && d.ldq >= d.K && d.ldp % 8 == 0 && d.ldq % 8 == 0,
                      "gemm desc %d: ldp=%d ldq=%d K=%d", i, d.ldp, d.ldq, d.K);
-        MUON_REQUIRE(!d.D || (d.ldd >= d.colsn), "gemm desc %d: ldd=%d < cols %d", i, d.ldd, d.colsn);
-        MUON_REQUIRE(!(d.C || d.C2) || d.ldc >= d.colsn, "gemm desc %d: ldc=%d < cols %d", i, d.ldc, d.colsn);
-        MUON_REQUIRE(!(d.CT || d.C2T) || (d.ldct >= d.rows && d.ldct % 4 == 0),
+        MUON_REQUIRE(!d.D || (d.ldd >= d.colsn && d.ldd % 4 == 0), "gemm desc %d: ldd=%d cols %d", i, d.ldd, d.colsn);
+        MUON_REQUIRE(!(d.C || d.C2) || (d.ldc >= d.colsn && d.ldc % 8 == 0), "gemm desc %d: ldc=%d cols %d", i, d.ldc, d.colsn);
+        MUON_REQUIRE(!(d.CT || d.C2T) || (d.ldct >= d.rows && d.ldct % 8 == 0),
                      "gemm desc %d: ldct=%d rows=%d", i, d.ldct, d.rows);
         MUON_REQUIRE((reinterpret_cast<uintptr_t>(d.P) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.Q) % 16) == 0 &&
-                         (reinterpret_cast<uintptr_t>(d.CT) % 8) == 0 && (reinterpret_cast<uintptr_t>(d.C2T) % 8) == 0,
+                         (reinterpret_cast<uintptr_t>(d.C) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.C2) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(d.CT) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.C2T) % 16) == 0 &&
+                         (reinterpret_cast<uintptr_t>(d.D) % 8) == 0,
                      "gemm desc %d: misaligned pointer", i);
         MUON_REQUIRE(!(d.C2 && !d.C) && !(d.C2T && !d.CT), "gemm desc %d: scaled copy needs its primary output", i);
     }
@@ -247,12 +481,15 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJ
         const MuonTileJob& t = jobs[j];
         MUON_REQUIRE(t.desc >= 0 && t.desc < ndesc, "job %d: desc %d out of range", j, t.desc);
         const MuonGemmDesc& d = descs[t.desc];
-        MUON_REQUIRE(t.i0 >= 0 && t.j0 >= 0 && t.i0 % T == 0 && t.j0 % T == 0 && t.i0 + T <= d.rows &&
-                         t.j0 + T <= d.colsn,
+        MUON_REQUIRE(t.i0 >= 0 && t.j0 >= 0 && t.i0 % TR == 0 && t.j0 % TC == 0 && t.i0 + TR <= d.rows &&
+                         t.j0 + TC <= d.colsn,
                      "job %d: tile (%d,%d) outside %dx%d", j, t.i0, t.j0, d.rows, d.colsn);
         MUON_REQUIRE(t.diag == 0 || t.diag == 1, "job %d: diag=%d", j, t.diag);
-        MUON_REQUIRE(!(d.CT == d.C && d.C) || (t.j0 >= t.i0 && t.diag == (t.i0 == t.j0)),
-                     "job %d: mirrored GEMM needs j0 >= i0 and diag set on the diagonal", j);
+        // mirrored GEMM: only tiles whose column block is on or above the row block, and tiles
+        // inside a diagonal TR x TR block (stored directly, never mirrored) are flagged
+        const int cblk = t.j0 / TR * TR;
+        MUON_REQUIRE(!(d.CT == d.C && d.C) || (cblk >= t.i0 && t.diag == (cblk == t.i0)),
+                     "job %d: mirrored GEMM needs its column block >= row block and diag set on the diagonal block", j);
     }
     return MUON_AMD_OK;
 }
@@ -262,37 +499,11 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
                      void* stream) {
     MUON_REQUIRE(descs_dev && jobs_dev, "ns_gemm: null table");
     MUON_REQUIRE(njobs > 0, "ns_gemm: njobs=%d", njobs);
-    MUON_REQUIRE(tile_class == 0 || tile_class == 1, "ns_gemm: unknown tile class %d", tile_class);
-    const int rt = (flags & MUON_AMD_ROUND_REFERENCE) ? 1 : 0;
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "ns_gemm: unknown tile class %d", tile_class);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (tile_class == 0) {
-        auto kern = ns_gemm_kernel<128, 128, 2, 2, 2>;
-        static bool attr_set = false;
-        if (!attr_set) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    static_cast<int>(kTileClasses[0].lds_bytes)) != hipSuccess) {
-                set_error("ns_gemm: cannot raise dynamic LDS to %zu bytes", kTileClasses[0].lds_bytes);
-                return MUON_AMD_ELAUNCH;
-            }
-            attr_set = true;
-        }
-        hipLaunchKernelGGL(kern, dim3(njobs), dim3(kTileClasses[0].threads), kTileClasses[0].lds_bytes, s,
-                           descs_dev, jobs_dev, alpha, beta, gamma, rt);
-    } else {
-        auto kern = ns_gemm_kernel<256, 256, 2, 4, 1>;
-        static bool attr_set = false;
-        if (!attr_set) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    static_cast<int>(kTileClasses[1].lds_bytes)) != hipSuccess) {
-                set_error("ns_gemm: cannot raise dynamic LDS to %zu bytes", kTileClasses[1].lds_bytes);
-                return MUON_AMD_ELAUNCH;
-            }
-            attr_set = true;
-        }
-        hipLaunchKernelGGL(kern, dim3(njobs), dim3(kTileClasses[1].threads), kTileClasses[1].lds_bytes, s,
-                           descs_dev, jobs_dev, alpha, beta, gamma, rt);
-    }
-    return check_launch("ns_gemm");
+    if (tile_class == 0) return launch_gemm<Cfg0>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, s);
+    return launch_gemm<Cfg1>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, s);
 }
+
 
 }  // extern "C"

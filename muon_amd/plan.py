@@ -12,6 +12,7 @@ which the iteration does not touch before the normalise kernel has consumed it.
 """
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass, field
 from functools import lru_cache
 
@@ -20,19 +21,27 @@ import numpy as np
 from . import _lib
 
 NS_COEFFS = (3.4445, -4.7750, 2.0315)   # reference muon.py:276
-TILE_EDGE = {0: 128, 1: 256}            # must match muon_amd_gemm_tile()
+TILE_DIMS = {0: (128, 128), 1: (256, 256)}   # must match muon_amd_gemm_tile_rows/cols()
+# output tiles (rows, cols) of one XCD-resident super-block: as many tiles as an XCD holds workgroups
+SUPER_DIMS = {0: (8, 8), 1: (4, 8)}
 EW_BLOCK_ELEMS = 8192                   # must match muon_amd_elementwise_block_elems()
 NT_TILE = 64                            # must match muon_amd_normalize_tile()
 N_XCD = 8                               # workgroups are dealt round-robin to the 8 XCDs
-SUPER_I, SUPER_J = 4, 8                 # output tiles per XCD-resident super-block
+# Workspace rows may be made this many elements longer than the padded width (a knob for
+# measurements: on MI355X a power-of-two row pitch measured no slower than a padded one).
+LD_PAD = int(os.environ.get("MUON_AMD_LD_PAD", "0"))
 _ALIGN = 256
 
 PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST = range(5)
 
 
 def tile_class_for(m: int) -> int:
-    """256-wide tiles once the short side fills them; 128-wide tiles below that."""
+    """256-row tiles once the short side fills them; 128 x 128 tiles below that."""
     return 1 if m >= 1024 else 0
+
+
+def pad_unit(tile_class: int) -> int:
+    return max(TILE_DIMS[tile_class])
 
 
 def _round_up(x: int, q: int) -> int:
@@ -52,6 +61,14 @@ class MatLayout:
     off: dict = field(default_factory=dict)   # byte offsets of X, XT0, XT1, A, B, CA
 
     @property
+    def ldn(self) -> int:     # leading dimension of X (rows of length np_)
+        return self.np_ + LD_PAD
+
+    @property
+    def ldm(self) -> int:     # leading dimension of X^T, A, B, c*A (rows of length mp)
+        return self.mp + LD_PAD
+
+    @property
     def rows_p(self) -> int:
         return self.mp if self.wide else self.np_
 
@@ -64,21 +81,23 @@ class MatLayout:
         return self.rows * self.cols
 
 
-def matrix_workspace_bytes(rows: int, cols: int, tile: int) -> int:
+def matrix_workspace_bytes(rows: int, cols: int, unit: int) -> int:
     m, n = min(rows, cols), max(rows, cols)
-    mp, np_ = _round_up(m, tile), _round_up(n, tile)
-    return 3 * _round_up(mp * np_ * 2, _ALIGN) + 3 * _round_up(mp * mp * 2, _ALIGN)
+    mp, np_ = _round_up(m, unit), _round_up(n, unit)
+    return (_round_up(mp * (np_ + LD_PAD) * 2, _ALIGN) + 2 * _round_up(np_ * (mp + LD_PAD) * 2, _ALIGN) +
+            3 * _round_up(mp * (mp + LD_PAD) * 2, _ALIGN))
 
 
 @lru_cache(maxsize=256)
-def _tile_order(mt: int, nt: int, sym: bool):
-    """Tiles of an mt x nt grid (upper triangle if sym) in super-block order."""
+def _tile_order(mt: int, nt: int, sym: bool, ratio: int, super_i: int, super_j: int):
+    """Tiles of an mt x nt grid in super-block order.  `ratio` = tile rows / tile cols; with sym
+    only tiles whose column block (j // ratio) is on or above their row block are kept."""
     ti, tj = [], []
-    for bi in range(0, mt, SUPER_I):
-        for bj in range(0, nt, SUPER_J):
-            for i in range(bi, min(bi + SUPER_I, mt)):
-                for j in range(bj, min(bj + SUPER_J, nt)):
-                    if sym and j < i:
+    for bi in range(0, mt, super_i):
+        for bj in range(0, nt, super_j):
+            for i in range(bi, min(bi + super_i, mt)):
+                for j in range(bj, min(bj + super_j, nt)):
+                    if sym and j // ratio < i:
                         continue
                     ti.append(i)
                     tj.append(j)
@@ -99,7 +118,8 @@ class ChunkPlan:
     def __init__(self, mats, tile_class: int, steps: int, reference_rounding: bool):
         # mats: list of (index, rows, cols)
         self.tile_class = tile_class
-        self.tile = TILE_EDGE[tile_class]
+        self.tile_rows, self.tile_cols = TILE_DIMS[tile_class]
+        self.tile = pad_unit(tile_class)          # padding unit of the chunk
         self.steps = steps
         self.reference_rounding = reference_rounding
         T = self.tile
@@ -108,9 +128,10 @@ class ChunkPlan:
         for index, rows, cols in mats:
             m, n = min(rows, cols), max(rows, cols)
             lay = MatLayout(index, rows, cols, m, n, _round_up(m, T), _round_up(n, T), rows <= cols)
-            xb = _round_up(lay.mp * lay.np_ * 2, _ALIGN)
-            ab = _round_up(lay.mp * lay.mp * 2, _ALIGN)
-            for name, nbytes in (("X", xb), ("XT0", xb), ("XT1", xb), ("A", ab), ("B", ab), ("CA", ab)):
+            xb = _round_up(lay.mp * lay.ldn * 2, _ALIGN)
+            tb = _round_up(lay.np_ * lay.ldm * 2, _ALIGN)
+            ab = _round_up(lay.mp * lay.ldm * 2, _ALIGN)
+            for name, nbytes in (("X", xb), ("XT0", tb), ("XT1", tb), ("A", ab), ("B", ab), ("CA", ab)):
                 lay.off[name] = off
                 off += nbytes
             self.layouts.append(lay)
@@ -133,17 +154,19 @@ class ChunkPlan:
 
     # ---- tile job lists -----------------------------------------------------------------
     def _jobs(self, sym: bool) -> np.ndarray:
-        T = self.tile
+        TR, TC = self.tile_rows, self.tile_cols
+        ratio = TR // TC
+        si, sj = SUPER_DIMS[self.tile_class]
         parts = []
         for k, lay in enumerate(self.layouts):
-            mt = lay.mp // T
-            nt = mt if sym else lay.np_ // T
-            ti, tj = _tile_order(mt, nt, sym)
+            mt = lay.mp // TR
+            nt = (lay.mp if sym else lay.np_) // TC
+            ti, tj = _tile_order(mt, nt, sym, ratio, si, sj)
             j = np.zeros(len(ti), dtype=_lib.TILE_JOB)
             j["desc"] = k
-            j["i0"] = ti * T
-            j["j0"] = tj * T
-            j["diag"] = (ti == tj).astype(np.int32) if sym else 0
+            j["i0"] = ti * TR
+            j["j0"] = tj * TC
+            j["diag"] = (ti == tj // ratio).astype(np.int32) if sym else 0
             parts.append(j)
         logical = np.concatenate(parts)
         return np.ascontiguousarray(logical[xcd_permutation(len(logical))])
@@ -162,32 +185,32 @@ class ChunkPlan:
             mp, np_ = lay.mp, lay.np_
             s = d[PH_SYRK, k]
             s["P"] = s["Q"] = p["X"]
-            s["ldp"] = s["ldq"] = np_
+            s["ldp"] = s["ldq"] = lay.ldn
             s["K"] = np_
             s["C"] = s["CT"] = p["A"]
             if self.reference_rounding:
                 s["C2"] = s["C2T"] = p["CA"]
-            s["ldc"] = s["ldct"] = mp
+            s["ldc"] = s["ldct"] = lay.ldm
             s["rows"] = s["colsn"] = mp
             q = d[PH_POLY, k]
             q["P"] = p["CA"] if self.reference_rounding else p["A"]
             q["Q"] = q["D"] = p["A"]
-            q["ldp"] = q["ldq"] = q["ldd"] = mp
+            q["ldp"] = q["ldq"] = q["ldd"] = lay.ldm
             q["K"] = mp
             q["C"] = q["CT"] = p["B"]
-            q["ldc"] = q["ldct"] = mp
+            q["ldc"] = q["ldct"] = lay.ldm
             q["rows"] = q["colsn"] = mp
             for ph, src, dst in ((PH_UPD_EVEN, "XT0", "XT1"), (PH_UPD_ODD, "XT1", "XT0")):
                 u = d[ph, k]
                 u["P"] = p["B"]
-                u["ldp"] = mp
+                u["ldp"] = lay.ldm
                 u["Q"] = p[src]
-                u["ldq"] = mp
+                u["ldq"] = lay.ldm
                 u["K"] = mp
                 u["D"] = u["C"] = p["X"]
-                u["ldd"] = u["ldc"] = np_
+                u["ldd"] = u["ldc"] = lay.ldn
                 u["CT"] = p[dst]
-                u["ldct"] = mp
+                u["ldct"] = lay.ldm
                 u["rows"] = mp
                 u["colsn"] = np_
             last = d[PH_UPD_LAST, k]
@@ -218,6 +241,8 @@ class ChunkPlan:
             r["denom"] = base + self.off_denoms + 4 * k
             r["rows"], r["cols"] = lay.rows, lay.cols
             r["rows_p"], r["cols_p"] = lay.rows_p, lay.cols_p
+            r["ld_direct"] = lay.ldn if lay.wide else lay.ldm
+            r["ld_transp"] = lay.ldm if lay.wide else lay.ldn
             r["part_begin"] = self.block_prefix[k]
             r["part_end"] = self.block_prefix[k + 1]
             r["scale"] = 1.0
@@ -244,7 +269,7 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
     for i in order:
         rows, cols = shapes[i]
         tc = tile_class_for(min(rows, cols))
-        need = matrix_workspace_bytes(rows, cols, TILE_EDGE[tc])
+        need = matrix_workspace_bytes(rows, cols, pad_unit(tc))
         if cur and (tc != cur_class or cur_bytes + need > workspace_cap):
             chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding))
             cur, cur_bytes = [], 0

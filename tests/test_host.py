@@ -27,15 +27,16 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
     lib = _lib.load()
     assert lib.muon_amd_abi_version() == 1
-    assert lib.muon_amd_gemm_tile(0) == plan.TILE_EDGE[0] and lib.muon_amd_gemm_tile(1) == plan.TILE_EDGE[1]
-    assert lib.muon_amd_gemm_tile(7) < 0 and b"tile class" in lib.muon_amd_last_error()
+    for tc, (tr, tcol) in plan.TILE_DIMS.items():
+        assert (lib.muon_amd_gemm_tile_rows(tc), lib.muon_amd_gemm_tile_cols(tc)) == (tr, tcol)
+    assert lib.muon_amd_gemm_tile_rows(7) < 0 and b"tile class" in lib.muon_amd_last_error()
     assert lib.muon_amd_elementwise_block_elems() == plan.EW_BLOCK_ELEMS
     assert lib.muon_amd_normalize_tile() == plan.NT_TILE
 
 
 def test_struct_layouts_match_the_library():
     lib = _lib.load()
-    assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 112
+    assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 120
     assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 88
     assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 16
     assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 48
@@ -70,23 +71,32 @@ def test_plans_validate_and_cover_every_tile_once(ref):
             jobs = c.sym_jobs if ph < 2 else c.full_jobs
             rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class)
             assert rc == 0, lib.muon_amd_last_error()
+        TR, TC = c.tile_rows, c.tile_cols
         for k, l in enumerate(c.layouts):
-            mt, nt = l.mp // T, l.np_ // T
+            mt, nt, ratio = l.mp // TR, l.np_ // TC, TR // TC
             sj = c.sym_jobs[c.sym_jobs["desc"] == k]
-            got = sorted(zip((sj["i0"] // T).tolist(), (sj["j0"] // T).tolist()))
-            assert got == [(i, j) for i in range(mt) for j in range(i, mt)]
-            assert np.array_equal(sj["diag"], (sj["i0"] == sj["j0"]).astype(np.int32))
+            got = sorted(zip((sj["i0"] // TR).tolist(), (sj["j0"] // TC).tolist()))
+            assert got == [(i, j) for i in range(mt) for j in range(i * ratio, l.mp // TC)]
+            assert np.array_equal(sj["diag"], (sj["i0"] // TR == sj["j0"] // TR).astype(np.int32))
+            # direct tiles plus mirrors of the off-diagonal-block tiles cover the matrix exactly once
+            cover = np.zeros((l.mp // TC, l.mp // TC), dtype=int)
+            for i0, j0, dg in zip(sj["i0"].tolist(), sj["j0"].tolist(), sj["diag"].tolist()):
+                cover[i0 // TC:(i0 + TR) // TC, j0 // TC] += 1
+                if not dg:
+                    cover[j0 // TC, i0 // TC:(i0 + TR) // TC] += 1
+            assert (cover == 1).all()
             fj = c.full_jobs[c.full_jobs["desc"] == k]
-            got = sorted(zip((fj["i0"] // T).tolist(), (fj["j0"] // T).tolist()))
+            got = sorted(zip((fj["i0"] // TR).tolist(), (fj["j0"] // TC).tolist()))
             assert got == [(i, j) for i in range(mt) for j in range(nt)]
             assert l.mp % T == 0 and l.np_ % T == 0 and l.mp >= l.m and l.np_ >= l.n
             assert l.wide == (l.rows <= l.cols)
         # workspace regions do not overlap and stay inside the chunk's workspace
         regions = []
         for l in c.layouts:
-            xb, ab = l.mp * l.np_ * 2, l.mp * l.mp * 2
+            size = {"X": l.mp * l.ldn * 2, "XT0": l.np_ * l.ldm * 2, "XT1": l.np_ * l.ldm * 2,
+                    "A": l.mp * l.ldm * 2, "B": l.mp * l.ldm * 2, "CA": l.mp * l.ldm * 2}
             for name in ("X", "XT0", "XT1", "A", "B", "CA"):
-                regions.append((l.off[name], l.off[name] + (xb if name.startswith("X") else ab)))
+                regions.append((l.off[name], l.off[name] + size[name]))
         regions += [(c.off_partials, c.off_partials + 4 * c.nblocks), (c.off_denoms, c.off_denoms + 4 * c.nmat)]
         regions.sort()
         assert all(a[1] <= b[0] for a, b in zip(regions, regions[1:])) and regions[-1][1] <= c.workspace_bytes
@@ -110,7 +120,7 @@ def test_validation_catches_a_bad_table():
     gd["K"] = 100                            # not a multiple of the k-block
     assert lib.muon_amd_validate_gemm(_lib.host_ptr(gd), 1, _lib.host_ptr(c.sym_jobs), len(c.sym_jobs), c.tile_class) == -1
     low = c.sym_jobs.copy()
-    low["i0"][0], low["j0"][0] = 128, 0      # below the diagonal of a mirrored GEMM
+    low["i0"][0], low["j0"][0] = c.tile_rows, 0      # below the diagonal of a mirrored GEMM
     assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[0]), 1, _lib.host_ptr(low), len(low), c.tile_class) == -1
 
 
