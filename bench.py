@@ -197,6 +197,9 @@ def main():
     ap.add_argument("--workload", default="llama3-8b", choices=["llama3-8b", "gpt2-124m", "conv"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary GPT-2 measurement")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="first run one plain 1 GiB device-to-device copy kernel (a known-size reference "
+                         "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the Muon update shards "
@@ -207,6 +210,12 @@ def main():
     steps = args.steps if args.steps is not None else dsteps
     warmup = args.warmup if args.warmup is not None else dwarm
 
+    if args.copy_probe:
+        a = torch.ones(1 << 28, dtype=torch.float32, device="cuda:0")      # 1 GiB
+        b = torch.empty_like(a)
+        b.copy_(a)                                                            # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del a, b
     res = run_optimizer_workload(args.workload, steps, warmup, seed=1234 + 4)
     kernels, gemm_work, gemm_ms, gemm_n = summarize_kernels(res["per_label"])
     ew_bytes = sum(w for l, (w, ms, n) in res["per_label"].items() if not l.startswith("ns_gemm"))

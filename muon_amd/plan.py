@@ -104,11 +104,23 @@ def _tile_order(mt: int, nt: int, sym: bool, ratio: int, super_i: int, super_j: 
     return np.asarray(ti, dtype=np.int32), np.asarray(tj, dtype=np.int32)
 
 
-def xcd_permutation(njobs: int) -> np.ndarray:
-    """physical block b runs logical job perm[b]: XCD x = b % 8 walks a contiguous logical range,
-    so the 32 workgroups resident on one XCD share operand panels in that XCD's L2."""
-    seg = -(-njobs // N_XCD)
-    idx = np.arange(N_XCD * seg, dtype=np.int64).reshape(N_XCD, seg).T.reshape(-1)
+XCD_MODE = os.environ.get("MUON_AMD_XCD_MODE", "interleave")
+
+
+def xcd_permutation(njobs: int, group: int = 32) -> np.ndarray:
+    """physical block b runs logical job perm[b].  Block b lands on XCD b % 8, as slot b // 8 of
+    that XCD.  Consecutive groups of `group` logical jobs (one super-block: as many tiles as an XCD
+    holds workgroups) are dealt round-robin to the XCDs: the workgroups resident on one XCD share
+    operand panels in its L2, and the eight XCDs work on neighbouring super-blocks of the same
+    matrix at the same time, so a panel one XCD pulled from HBM is found in the memory-side cache
+    by the others."""
+    if XCD_MODE == "segment":      # each XCD walks one contiguous eighth of the list
+        seg = -(-njobs // N_XCD)
+        idx = np.arange(N_XCD * seg, dtype=np.int64).reshape(N_XCD, seg).T.reshape(-1)
+        return idx[idx < njobs]
+    b = np.arange(-(-njobs // (N_XCD * group)) * N_XCD * group, dtype=np.int64)
+    x, s = b % N_XCD, b // N_XCD
+    idx = ((s // group) * N_XCD + x) * group + (s % group)
     return idx[idx < njobs]
 
 
@@ -169,7 +181,7 @@ class ChunkPlan:
             j["diag"] = (ti == tj // ratio).astype(np.int32) if sym else 0
             parts.append(j)
         logical = np.concatenate(parts)
-        return np.ascontiguousarray(logical[xcd_permutation(len(logical))])
+        return np.ascontiguousarray(logical[xcd_permutation(len(logical), si * sj)])
 
     # ---- descriptor tables -----------------------------------------------------------------
     def result_buffer(self, lay: MatLayout) -> str:

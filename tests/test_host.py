@@ -125,11 +125,13 @@ def test_validation_catches_a_bad_table():
 
 
 def test_xcd_permutation_and_result_buffer():
-    for n in (1, 7, 8, 9, 136, 1000):
-        p = plan.xcd_permutation(n)
-        assert sorted(p.tolist()) == list(range(n))
-    p = plan.xcd_permutation(64)                 # block b runs on XCD b % 8: contiguous logical range per XCD
-    assert p[:8].tolist() == [0, 8, 16, 24, 32, 40, 48, 56] and p[8] == 1
+    for n in (1, 7, 8, 9, 136, 1000, 4352):
+        for group in (32, 64):
+            p = plan.xcd_permutation(n, group)
+            assert sorted(p.tolist()) == list(range(n))
+    p = plan.xcd_permutation(512, 32)            # block b runs on XCD b % 8, slot b // 8
+    assert p[:8].tolist() == [0, 32, 64, 96, 128, 160, 192, 224] and p[8] == 1      # a 32-job group per XCD
+    assert p[256:264].tolist() == [256, 288, 320, 352, 384, 416, 448, 480]           # next round of groups
     for steps, want_tall in ((0, "XT0"), (1, "XT1"), (2, "XT0"), (5, "XT1")):
         c = plan.ChunkPlan([(0, 300, 100), (1, 100, 300)], 0, steps, True)
         assert c.result_buffer(c.layouts[0]) == want_tall and c.result_buffer(c.layouts[1]) == "X"
