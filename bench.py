@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 
 
 # ------------------------------------------------------------------------------------------
-# workloads (BASELINE.json configs)
+# workloads: the benchmark configurations (parameter sets of GPT-2-small, Llama-3-8B, a CIFAR ConvNet)
 # ------------------------------------------------------------------------------------------
 def workload_shapes(name):
     """-> (muon [(shape, count)], adam [(shape, count)], grad_std, default_steps, default_warmup)"""
@@ -203,7 +203,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the Muon update shards "
-                 "by matrix across ranks; see DESIGN.md). Run with --gpus 1.")
+                 "by matrix across ranks, which is not part of this library). Run with --gpus 1.")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X GPU")
     _, _, _, dsteps, dwarm = workload_shapes(args.workload)

@@ -24,6 +24,8 @@ NS_COEFFS = (3.4445, -4.7750, 2.0315)   # reference muon.py:276
 TILE_DIMS = {0: (128, 128), 1: (256, 256)}   # must match muon_amd_gemm_tile_rows/cols()
 # output tiles (rows, cols) of one XCD-resident super-block: as many tiles as an XCD holds workgroups
 SUPER_DIMS = {0: (8, 8), 1: (4, 8)}
+if os.environ.get("MUON_AMD_SUPER"):     # measurement knob: "rows,cols" of the 256 x 256 class super-block
+    SUPER_DIMS[1] = tuple(int(v) for v in os.environ["MUON_AMD_SUPER"].split(","))
 EW_BLOCK_ELEMS = 8192                   # must match muon_amd_elementwise_block_elems()
 NT_TILE = 64                            # must match muon_amd_normalize_tile()
 N_XCD = 8                               # workgroups are dealt round-robin to the 8 XCDs
@@ -35,9 +37,12 @@ _ALIGN = 256
 PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST = range(5)
 
 
+BIG_TILE_MIN_M = int(os.environ.get("MUON_AMD_BIG_TILE_MIN_M", "1024"))
+
+
 def tile_class_for(m: int) -> int:
-    """256-row tiles once the short side fills them; 128 x 128 tiles below that."""
-    return 1 if m >= 1024 else 0
+    """256 x 256 tiles once the short side is long enough to fill them; 128 x 128 tiles below."""
+    return 1 if m >= BIG_TILE_MIN_M else 0
 
 
 def pad_unit(tile_class: int) -> int:
@@ -181,7 +186,8 @@ class ChunkPlan:
             j["diag"] = (ti == tj // ratio).astype(np.int32) if sym else 0
             parts.append(j)
         logical = np.concatenate(parts)
-        return np.ascontiguousarray(logical[xcd_permutation(len(logical), si * sj)])
+        group = int(os.environ.get("MUON_AMD_XCD_GROUP", si * sj))      # measurement knob
+        return np.ascontiguousarray(logical[xcd_permutation(len(logical), group)])
 
     # ---- descriptor tables -----------------------------------------------------------------
     def result_buffer(self, lay: MatLayout) -> str:

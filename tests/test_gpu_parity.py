@@ -2,7 +2,7 @@
 seeded inputs, against the committed golden fixtures, and through size-independent properties
 at the full benchmark sizes.
 
-Tolerances (BASELINE.json north_star): Newton-Schulz output within 2e-2 relative Frobenius error
+Tolerances of the build's acceptance contract: Newton-Schulz output within 2e-2 relative Frobenius error
 of the reference bf16 result and 3e-2 of the fp32 oracle; parameters within 1e-3 after a step;
 auxiliary Adam within 1e-5.
 """
@@ -218,7 +218,7 @@ def _set_grads(cpu, gpu, std):
 
 
 def test_config1_single_device_muon_step(M):
-    """BASELINE config 1: one 768x3072 weight, lr .02, wd .01, momentum .95, one step."""
+    """Benchmark configuration 1: one 768x3072 weight, lr .02, wd .01, momentum .95, one step."""
     cpu, gpu = _clone_params([(768, 3072)], 0.02, 1235)
     _set_grads(cpu, gpu, 1e-3)
     oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95)
@@ -232,7 +232,7 @@ def test_config1_single_device_muon_step(M):
 
 
 def test_gpt2_like_aux_adam_steps(M):
-    """BASELINE config 2 at 2 layers (same matrix shapes, embeddings cut to 4096 rows), 4 steps."""
+    """Benchmark configuration 2 (GPT-2-small) at 2 layers (same matrix shapes, embeddings cut to 4096 rows), 4 steps."""
     muon_shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 2
     adam_shapes = [(4096, 768), (1024, 768)] + [(768,)] * 5
     cpu_m, gpu_m = _clone_params(muon_shapes, 0.02, 1236)
@@ -253,7 +253,7 @@ def test_gpt2_like_aux_adam_steps(M):
 
 
 def test_conv_and_odd_shapes_step(M):
-    """BASELINE config 5: conv filters flattened to 2-D, extreme aspect ratios, tiny Adam tensors."""
+    """Benchmark configuration 5 (CIFAR ConvNet): conv filters flattened to 2-D, extreme aspect ratios, tiny Adam tensors."""
     muon_shapes = [(64, 24, 3, 3), (256, 64, 3, 3), (256, 256, 3, 3), (256, 256, 3, 3), (512, 256, 3, 3),
                    (512, 512, 3, 3), (128, 16384), (16384, 128)]
     adam_shapes = [(24, 3, 2, 2), (10, 512)]
