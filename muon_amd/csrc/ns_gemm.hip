@@ -56,8 +56,21 @@ __device__ __forceinline__ void dma16(const uint16_t* gptr, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n"
                  :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
-// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained); n < 16.
-#define NS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | (n))
+// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained); n < 64 (bits 3:0 and 15:14).
+#define NS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+
+// Wait until at most min(n, H) half-stages (DPH DMA instructions each) of this wave are pending.
+template <int DPH, int H>
+struct WaitHalves {
+    static __device__ __forceinline__ void run(int n) {
+        if (n >= H) NS_WAIT_VMCNT(H * DPH);
+        else WaitHalves<DPH, H - 1>::run(n);
+    }
+};
+template <int DPH>
+struct WaitHalves<DPH, 0> {
+    static __device__ __forceinline__ void run(int) { NS_WAIT_VMCNT(0); }
+};
 
 // ---------------------------------------------------------------------------------------------
 // Epilogue helpers
@@ -195,15 +208,18 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
     }
 
     if (do_d) {
-        constexpr int CPR = WN / 8, RPI = 64 / CPR;     // 16-byte chunks per row, rows per wave store
+        // 16-byte chunks per row, whole rows per wave-wide store (lanes beyond RPI rows idle)
+        constexpr int CPR = WN / 8, RPI = 64 / CPR;
         const int r = lane / CPR, ch = lane % CPR;
 #pragma unroll
-        for (int it = 0; it < WM / RPI; ++it) {
+        for (int it = 0; it < (WM + RPI - 1) / RPI; ++it) {
             const int row = it * RPI + r;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
-            const size_t off = static_cast<size_t>(row0 + row) * d.ldc + col0 + ch * 8;
-            gstore16(d.C + off, v);
-            if (d.C2) gstore16(d.C2 + off, scale_bf16x8(v, gamma));
+            if (r < RPI && row < WM) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
+                const size_t off = static_cast<size_t>(row0 + row) * d.ldc + col0 + ch * 8;
+                gstore16(d.C + off, v);
+                if (d.C2) gstore16(d.C2 + off, scale_bf16x8(v, gamma));
+            }
         }
     }
     if (do_t) {
@@ -221,12 +237,14 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
         constexpr int CPR = WM / 8, RPI = 64 / CPR;
         const int r = lane / CPR, ch = lane % CPR;
 #pragma unroll
-        for (int it = 0; it < WN / RPI; ++it) {
+        for (int it = 0; it < (WN + RPI - 1) / RPI; ++it) {
             const int row = it * RPI + r;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
-            const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + ch * 8;
-            gstore16(d.CT + off, v);
-            if (d.C2T) gstore16(d.C2T + off, scale_bf16x8(v, gamma));
+            if (r < RPI && row < WN) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
+                const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + ch * 8;
+                gstore16(d.CT + off, v);
+                if (d.C2T) gstore16(d.C2T + off, scale_bf16x8(v, gamma));
+            }
         }
     }
 }
@@ -234,17 +252,15 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 // ---------------------------------------------------------------------------------------------
 // The kernel
 // ---------------------------------------------------------------------------------------------
-// The LDS ring holds NHALF = 5 half-stages; a half-stage is the P rows or the Q rows of one
-// k-block (BT rows x 128 bytes).  Half-stages are issued in the order P0 Q0 P1 Q1 P2 ...; block kb
-// needs halves 2kb and 2kb+1.  While block kb is multiplied, half 2kb+2 (issued one iteration
-// earlier) and halves 2kb+3, 2kb+4 (issued at the top of this iteration into the two slots
-// block kb-1 vacated) are in flight, so the load pipe always has a queued request and every
-// request is a full 128-byte line.
-constexpr int NHALF = 5;
-
-template <int BT_, int WGM_, int WGN_, int MINB_>
+// The LDS ring holds NHALF half-stages; a half-stage is the P rows or the Q rows of one k-block
+// (BT rows x 128 bytes).  Half-stages are issued in the order P0 Q0 P1 Q1 P2 ...; block kb needs
+// halves 2kb and 2kb+1.  While block kb is multiplied, the halves up to 2kb+NHALF-3 (issued in
+// earlier iterations) and halves 2kb+NHALF-2, 2kb+NHALF-1 (issued during this iteration into the
+// two slots block kb-1 vacated) are in flight, so the load pipe always has queued requests and
+// every request is a full 128-byte line.  NHALF = 5 fills the 160 KB LDS for the 256 x 256 tile.
+template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_>
 struct GemmCfg {
-    static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_;
+    static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_, NHALF = NHALF_;
     static constexpr int NW = WGM * WGN, NT = NW * 64;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int HALF_BYTES = BT_ * ROW_BYTES;
@@ -253,7 +269,7 @@ struct GemmCfg {
     static constexpr size_t EPI_BYTES = static_cast<size_t>(NW) * epilogue_stage_bytes(WM, WN);
     static constexpr size_t LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
     static_assert(BT_ % (8 * NW) == 0, "DMA tiling");
-    static_assert(3 * DPH < 16, "vmcnt immediate");
+    static_assert((NHALF - 2) * DPH < 64 && NHALF >= 5, "vmcnt immediate / ring depth");
     static_assert(NW % 2 == 0, "swizzle parity assumes an even wave count");
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be MFMA tiles");
     static_assert(LDS_BYTES <= 163840, "LDS capacity of a gfx950 CU");
@@ -265,6 +281,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     float beta, float gamma, int flags) {
     constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
+    constexpr int NHALF = Cfg::NHALF;
     extern __shared__ __align__(16) uint16_t lds[];
     const MuonTileJob job = jobs[blockIdx.x];
     const MuonGemmDesc d = descs[job.desc];
@@ -313,74 +330,86 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
     const int nk = d.K / BK;
-    // prologue: halves 0..4 = P0 Q0 P1 Q1 P2
-    NS_ISSUE_HALF(srcp, 0, 0);
-    NS_ISSUE_HALF(srcq, 0, 1);
-    if (nk > 1) {
-        NS_ISSUE_HALF(srcp, 1, 2);
-        NS_ISSUE_HALF(srcq, 1, 3);
+    // prologue: halves 0 .. NHALF-1 = P0 Q0 P1 Q1 P2 ...
+#pragma unroll
+    for (int h = 0; h < NHALF; ++h) {
+        if (h < 2 * nk) {
+            if (h & 1) NS_ISSUE_HALF(srcq, h >> 1, h);
+            else NS_ISSUE_HALF(srcp, h >> 1, h);
+        }
     }
-    if (nk > 2) NS_ISSUE_HALF(srcp, 2, 4);
+
+    constexpr int KSTEPS = BK / 16;
+    constexpr int DPK = 2 * DPH / KSTEPS;                    // DMA instructions per k-step
+    static_assert(2 * DPH % KSTEPS == 0 && DPH % DPK == 0, "DMA instructions must spread evenly");
+    static_assert(DPK <= TM, "one DMA instruction per row of MFMAs");
+
+    // Block 0 has landed once only the younger prologue halves are pending.
+    WaitHalves<DPH, NHALF - 2>::run((2 * nk < NHALF ? 2 * nk : NHALF) - 2);
+    __syncthreads();
+
+    // Fragments are double buffered over k-steps ACROSS blocks: the ds_reads of the next k-step
+    // (the first one of block kb+1 included) are issued ahead of the MFMAs of the current one, so
+    // the matrix pipe never waits for LDS latency, not even right after the barrier.
+    bf16x8 af[2][TM], bfr[2][TN];
+#define NS_LOAD_FRAGS(buf_, pf_, qf_, ks_)                                                      \
+    do {                                                                                       \
+        _Pragma("unroll") for (int a_ = 0; a_ < TM; ++a_)                                      \
+            af[buf_][a_] = *reinterpret_cast<const bf16x8*>((pf_) + a_ * 32 * ROW_BYTES + koff[ks_]); \
+        _Pragma("unroll") for (int b_ = 0; b_ < TN; ++b_)                                      \
+            bfr[buf_][b_] = *reinterpret_cast<const bf16x8*>((qf_) + b_ * 32 * ROW_BYTES + koff[ks_]); \
+    } while (0)
+    NS_LOAD_FRAGS(0, pfrag, qfrag + HALF_BYTES, 0);
+
+    // The pair of halves being issued: created at the barrier of block kb (last k-step), its
+    // 2*DPH DMA instructions are spread over that k-step and the first KSTEPS-1 of block kb+1,
+    // one after each of the first DPK rows of MFMAs -- a burst right after the barrier would hold
+    // every wave in the memory-issue queue while the matrix pipe sits idle.
+    // NHALF odd: the first half of a pair is a Q half (needed one block earlier), the second P.
+    const uint16_t* const* dsrc[2] = {(NHALF & 1) ? srcq : srcp, (NHALF & 1) ? srcp : srcq};
+    uint32_t ddst[2] = {0, 0};
+    size_t dk[2] = {0, 0};
+    bool dgo[2] = {false, false};
 
     int sp = 0, sq = 1;                 // ring slots of the P and Q halves of block kb
     for (int kb = 0; kb < nk; ++kb) {
-        // halves 2kb and 2kb+1 have landed once only the younger halves are pending
-        if (kb == 0) {
-            if (nk > 2) NS_WAIT_VMCNT(3 * DPH);
-            else if (nk > 1) NS_WAIT_VMCNT(2 * DPH);
-            else NS_WAIT_VMCNT(0);
-        } else {
-            if (kb + 1 < nk) NS_WAIT_VMCNT(DPH);
-            else NS_WAIT_VMCNT(0);
-        }
-        __syncthreads();   // block kb visible to all waves; the two slots of block kb-1 are free
-        // halves 2kb+3 = Q(kb+1) and 2kb+4 = P(kb+2) go into the slots of halves 2kb-2, 2kb-1.
-        // Their 2*DPH DMA instructions are spread over the k-steps below, between the MFMAs: a
-        // burst right after the barrier would hold every wave in the memory-issue queue while
-        // the matrix pipe sits idle.
-        int s3 = sq + 2; s3 = s3 >= NHALF ? s3 - NHALF : s3;     // (2kb+3) % 5
-        int s4 = sp + 4; s4 = s4 >= NHALF ? s4 - NHALF : s4;     // (2kb+4) % 5
-        const bool issue_q = kb >= 1 && kb + 1 < nk;
-        const bool issue_p = kb >= 1 && kb + 2 < nk;
-        const uint16_t* const* dsrc[2] = {srcq, srcp};
-        const uint32_t ddst[2] = {dst0 + s3 * HALF_BYTES, dst0 + s4 * HALF_BYTES};
-        const size_t dk[2] = {static_cast<size_t>(kb + 1) * BK, static_cast<size_t>(kb + 2) * BK};
-        const bool dgo[2] = {issue_q, issue_p};
-        constexpr int KSTEPS = BK / 16;
-        constexpr int DPK = 2 * DPH / KSTEPS;                    // DMA instructions per k-step
-        static_assert(2 * DPH % KSTEPS == 0 && DPH % DPK == 0, "DMA instructions must spread evenly");
-
         const char* const pf = pfrag + sp * HALF_BYTES;
         const char* const qf = qfrag + sq * HALF_BYTES;
-        // fragments are double buffered: the ds_reads of k-step ks+1 are issued ahead of the
-        // MFMAs of k-step ks, so the matrix pipe never waits for LDS latency inside a block
-        bf16x8 af[2][TM], bfr[2][TN];
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
-            af[0][a] = *reinterpret_cast<const bf16x8*>(pf + a * 32 * ROW_BYTES + koff[0]);
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-            bfr[0][b] = *reinterpret_cast<const bf16x8*>(qf + b * 32 * ROW_BYTES + koff[0]);
+        int spn = sp + 2; spn = spn >= NHALF ? spn - NHALF : spn;
+        int sqn = sq + 2; sqn = sqn >= NHALF ? sqn - NHALF : sqn;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             const int cur = ks & 1, nxt = cur ^ 1;
             if (ks + 1 < KSTEPS) {
-#pragma unroll
-                for (int a = 0; a < TM; ++a)
-                    af[nxt][a] = *reinterpret_cast<const bf16x8*>(pf + a * 32 * ROW_BYTES + koff[ks + 1]);
-#pragma unroll
-                for (int b = 0; b < TN; ++b)
-                    bfr[nxt][b] = *reinterpret_cast<const bf16x8*>(qf + b * 32 * ROW_BYTES + koff[ks + 1]);
-                __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
+                NS_LOAD_FRAGS(nxt, pf, qf, ks + 1);
+            } else if (kb + 1 < nk) {
+                // Every fragment of block kb is in registers (the barrier waits for this wave's
+                // LDS reads).  Block kb+1 has landed once only the younger halves are pending;
+                // after the barrier it is visible to all waves and the two slots of block kb are
+                // free for the next pair of halves, 2kb+NHALF and 2kb+NHALF+1.
+                const int issued = 2 * nk < 2 * kb + NHALF ? 2 * nk : 2 * kb + NHALF;
+                WaitHalves<DPH, NHALF - 2>::run(issued - (2 * kb + 4));
+                __syncthreads();
+                const int h0 = 2 * kb + NHALF;
+                ddst[0] = dst0 + sp * HALF_BYTES;                // h0 % NHALF == 2kb % NHALF
+                ddst[1] = dst0 + sq * HALF_BYTES;
+                dk[0] = static_cast<size_t>(h0 >> 1) * BK;
+                dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;
+                dgo[0] = h0 < 2 * nk;
+                dgo[1] = h0 + 1 < 2 * nk;
+                NS_LOAD_FRAGS(nxt, pfrag + spn * HALF_BYTES, qfrag + sqn * HALF_BYTES, 0);
+            } else {
+                dgo[0] = dgo[1] = false;     // last block: nothing left to fetch
             }
+            __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
 #pragma unroll
             for (int a = 0; a < TM; ++a) {
 #pragma unroll
                 for (int b = 0; b < TN; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][a], bfr[cur][b], acc[a][b], 0, 0, 0);
-                // one DMA instruction after each of the first DPK rows of MFMAs of this k-step
                 if (a < DPK) {
-                    const int jj = ks * DPK + a;                 // 0 .. 2*DPH-1, Q half first
+                    // instruction jj of the current pair: the last k-step starts a pair
+                    const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;
                     const int h = jj / DPH, j = jj % DPH;
                     __builtin_amdgcn_sched_barrier(0);
                     if (dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024);
@@ -389,9 +418,10 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        sp += 2; sp = sp >= NHALF ? sp - NHALF : sp;
-        sq += 2; sq = sq >= NHALF ? sq - NHALF : sq;
+        sp = spn;
+        sq = sqn;
     }
+#undef NS_LOAD_FRAGS
 #undef NS_ISSUE_HALF
     __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
     char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
@@ -403,8 +433,12 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 // Tile classes: square output tile, waves, workgroups per CU.
 //   0: 128 x 128, 4 waves of 64 x 64, two workgroups per CU   (short side below 1024)
 //   1: 256 x 256, 8 waves of 128 x 64, one workgroup per CU   (large matrices)
-typedef GemmCfg<128, 2, 2, 2> Cfg0;
-typedef GemmCfg<256, 2, 4, 1> Cfg1;
+#ifndef NS_CFG0_MINB
+#define NS_CFG0_MINB 2
+#define NS_CFG0_NHALF 5
+#endif
+typedef GemmCfg<128, 2, 2, NS_CFG0_MINB, NS_CFG0_NHALF> Cfg0;
+typedef GemmCfg<256, 2, 4, 1, 5> Cfg1;
 constexpr int kNumTileClasses = 2;
 
 struct TileClass {
