@@ -44,8 +44,6 @@ class _MuonBase(torch.optim.Optimizer):
         require_gpu_tensor(p, "parameter")
         if p.dtype != torch.float32:
             raise NotImplementedError(f"muon_amd updates fp32 parameters; got {p.dtype}")
-        if not p.is_contiguous():
-            raise NotImplementedError("muon_amd needs contiguous parameters")
 
     @staticmethod
     def _grad_of(p):
@@ -54,35 +52,56 @@ class _MuonBase(torch.optim.Optimizer):
         g = p.grad
         if g.dtype != torch.float32 or g.is_sparse:
             raise NotImplementedError("muon_amd needs dense fp32 gradients")
-        if not g.is_contiguous():
-            g = p.grad = g.contiguous()
         return g
+
+    @staticmethod
+    def _dense(t, writebacks, written=True):
+        """The kernels address row-major memory.  A tensor with other strides (a transposed view
+        used as a parameter, say) goes through a contiguous copy that is copied back after the
+        launches; the reference takes any strides because torch does (muon.py:9-10, 98-99)."""
+        if t.is_contiguous():
+            return t
+        c = t.contiguous()
+        if written:
+            writebacks.append((t, c))
+        return c
+
+    @staticmethod
+    def _state_tensor(state, key, p):
+        t = state[key]
+        if t.dtype != torch.float32 or t.device != p.device or t.shape != p.shape:
+            raise NotImplementedError(f"{key} must be an fp32 tensor of the parameter's shape on its device")
+        return t
 
     def _muon_group_step(self, gi, group):
         params = [p for p in group["params"] if p.numel() > 0]
         if not params:
             return
-        grads, moms, shapes, scales = [], [], [], []
+        grads, moms, ptrs, shapes, scales, writebacks, keep = [], [], [], [], [], [], []
         for p in params:
             self._check_param(p)
             assert p.ndim >= 2                    # muon.py:275 (reached through muon.py:13)
             g = self._grad_of(p)
             state = self.state[p]
             if len(state) == 0:                   # muon.py:95-96
-                state["momentum_buffer"] = torch.zeros_like(p)
-            m = state["momentum_buffer"]
-            if m.dtype != torch.float32 or not m.is_contiguous() or m.device != p.device:
-                raise NotImplementedError("momentum_buffer must be a contiguous fp32 tensor on the parameter's device")
-            if p.ndim == 4:                       # muon.py:11-12
-                rows, cols = p.size(0), p.numel() // p.size(0)
-            elif p.ndim == 2:
-                rows, cols = p.shape
-            else:
-                raise NotImplementedError("muon_amd optimizers take 2-D matrices and 4-D conv filters")
-            shapes.append((rows, cols))
-            scales.append(max(1, p.size(-2) / p.size(-1)) ** 0.5)     # muon.py:14
-            grads.append(g.data_ptr())
-            moms.append(m.data_ptr())
+                state["momentum_buffer"] = torch.zeros_like(p, memory_format=torch.contiguous_format)
+            m = self._dense(self._state_tensor(state, "momentum_buffer", p), writebacks)
+            g = self._dense(g, writebacks, written=self._mutate_grad)
+            pc = self._dense(p, writebacks)
+            keep.append((g, m, pc))               # copies stay allocated until the launches are enqueued
+            if p.ndim == 4:                       # muon.py:11-12: conv filters are flattened
+                batch, rows, cols = 1, p.size(0), p.numel() // p.size(0)
+            else:                                 # muon.py:275, 282: leading dims are a batch
+                rows, cols = p.shape[-2:]
+                batch = p.numel() // (rows * cols)
+            scale = max(1, p.size(-2) / p.size(-1)) ** 0.5             # muon.py:14
+            for k in range(batch):
+                off = k * rows * cols * 4
+                shapes.append((rows, cols))
+                scales.append(scale)
+                grads.append(g.data_ptr() + off)
+                moms.append(m.data_ptr() + off)
+                ptrs.append(pc.data_ptr() + off)
         device = params[0].device
         key = (gi, device, tuple(shapes))
         eng = self._muon_engines.get(key)
@@ -90,38 +109,45 @@ class _MuonBase(torch.optim.Optimizer):
             self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
             eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes)
             self._muon_engines[key] = eng
-        n = len(params)
+        n = len(shapes)
         with torch.cuda.device(device):
-            eng.run(grads, moms, [p.data_ptr() for p in params], [0] * n, scales, [_lib.SRC_F32] * n,
+            eng.run(grads, moms, ptrs, [0] * n, scales, [_lib.SRC_F32] * n,
                     beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad,
                     eps=1e-7, lr=group["lr"], weight_decay=group["weight_decay"])
+            for dst, src in writebacks:           # stream ordered after the launches
+                dst.copy_(src)
 
     def _adam_group_step(self, gi, group):
-        by_step = {}
+        by_step, writebacks = {}, []
         for p in group["params"]:
             self._check_param(p)
             g = self._grad_of(p)
             state = self.state[p]
             if len(state) == 0:                   # muon.py:250-253
-                state["exp_avg"] = torch.zeros_like(p)
-                state["exp_avg_sq"] = torch.zeros_like(p)
+                state["exp_avg"] = torch.zeros_like(p, memory_format=torch.contiguous_format)
+                state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.contiguous_format)
                 state["step"] = 0
             state["step"] += 1                    # muon.py:254
             if p.numel() > 0:
-                by_step.setdefault(int(state["step"]), []).append((p, g, state))
+                item = (self._dense(p, writebacks), self._dense(g, writebacks, written=False),
+                        self._dense(self._state_tensor(state, "exp_avg", p), writebacks),
+                        self._dense(self._state_tensor(state, "exp_avg_sq", p), writebacks))
+                by_step.setdefault(int(state["step"]), []).append((p, item))
         for step, items in by_step.items():
             device = items[0][0].device
-            key = (gi, device, tuple(id(p) for p, _, _ in items))
+            key = (gi, device, tuple(id(p) for p, _ in items))
             eng = self._adam_engines.get(key)
             if eng is None:
-                eng = AdamGroupEngine([p.numel() for p, _, _ in items], device)
+                eng = AdamGroupEngine([p.numel() for p, _ in items], device)
                 self._adam_engines[key] = eng
             with torch.cuda.device(device):
-                eng.run([p.data_ptr() for p, _, _ in items], [g.data_ptr() for _, g, _ in items],
-                        [s["exp_avg"].data_ptr() for _, _, s in items],
-                        [s["exp_avg_sq"].data_ptr() for _, _, s in items], [0] * len(items),
+                eng.run([t[0].data_ptr() for _, t in items], [t[1].data_ptr() for _, t in items],
+                        [t[2].data_ptr() for _, t in items], [t[3].data_ptr() for _, t in items],
+                        [0] * len(items),
                         lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"],
                         eps=group["eps"], step=step)
+        for dst, src in writebacks:
+            dst.copy_(src)
 
     @staticmethod
     def _run_closure(closure):

@@ -341,3 +341,102 @@ def test_optimizer_behaviour_on_gpu(M):
     assert torch.equal(r.grad, g)
     with pytest.raises(AssertionError):
         M.SingleDeviceMuon([torch.nn.Parameter(torch.ones(8, device="cuda"))]).step()   # ndim >= 2
+
+
+# ------------------------------------------------------------------------------------------
+# parameter layouts beyond plain 2-D / conv: batched matrices, other strides, late groups,
+# checkpoints written in the reference's state layout
+# ------------------------------------------------------------------------------------------
+def test_batched_matrix_parameters_step(M):
+    """3-D and 5-D Muon parameters are batches of matrices over the leading dims (the iteration of
+    muon.py:275-291 is batched; only 4-D tensors are flattened, muon.py:11-12)."""
+    shapes = [(3, 64, 96), (2, 2, 3, 40, 24), (4, 130, 130)]
+    cpu, gpu = _clone_params(shapes, 0.02, 1301)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    for step in range(2):
+        _set_grads(cpu, gpu, 1e-2)
+        oc.step()
+        og.step()
+        for pc, pg in zip(cpu, gpu):
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 2e-3, (tuple(pc.shape), step)   # small matrices: see the golden-step test
+            np.testing.assert_allclose(og.state[pg]["momentum_buffer"].cpu().numpy(),
+                                       oc.state[pc]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-10)
+
+
+def test_non_contiguous_parameters_and_gradients_step(M):
+    """A transposed view as a parameter, a strided gradient, and an Adam tensor with a gap."""
+    torch.manual_seed(1302)
+    w = torch.randn(96, 160) * 0.02
+    e = torch.randn(50, 64) * 0.02
+    cpu_m = torch.nn.Parameter(w.clone().t())                 # 160 x 96, column-major
+    gpu_m = torch.nn.Parameter(_dev(w.clone()).t())
+    cpu_a = torch.nn.Parameter(e.clone()[:, ::2])             # 50 x 32, row stride 64, column stride 2
+    gpu_a = torch.nn.Parameter(_dev(e.clone())[:, ::2])
+    assert not gpu_m.is_contiguous() and not gpu_a.is_contiguous()
+    mk = lambda cls, pm, pa: cls([dict(params=[pm], use_muon=True, lr=0.02, weight_decay=0.01),
+                                  dict(params=[pa], use_muon=False, lr=3e-4, weight_decay=0.01)])
+    oc, og = mk(O.OracleSingleDeviceMuonWithAuxAdam, cpu_m, cpu_a), mk(M.SingleDeviceMuonWithAuxAdam, gpu_m, gpu_a)
+    for step in range(3):
+        gm = torch.randn(96, 160) * 1e-2
+        ga = torch.randn(50, 32) * 1e-2
+        cpu_m.grad, gpu_m.grad = gm.clone().t(), _dev(gm.clone()).t()          # strided gradient
+        cpu_a.grad, gpu_a.grad = ga.clone(), _dev(ga.clone())
+        oc.step()
+        og.step()
+        assert O.rel_fro(gpu_m.detach().cpu(), cpu_m.detach()) <= TOL_PARAM, step
+        np.testing.assert_allclose(gpu_a.detach().cpu().numpy(), cpu_a.detach().numpy(), rtol=TOL_ADAM, atol=1e-8)
+    assert gpu_m.stride() == (1, 160)                          # updated in place, layout kept
+    np.testing.assert_allclose(og.state[gpu_m]["momentum_buffer"].cpu().numpy(),
+                               oc.state[cpu_m]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-10)
+
+
+def test_add_param_group_after_first_step(M):
+    cpu, gpu = _clone_params([(64, 96), (48, 48), (33,)], 0.02, 1303)
+    mk = lambda cls, ps: cls([dict(params=[ps[0]], use_muon=True, lr=0.02, weight_decay=0.01)])
+    oc, og = mk(O.OracleSingleDeviceMuonWithAuxAdam, cpu), mk(M.SingleDeviceMuonWithAuxAdam, gpu)
+    _set_grads(cpu, gpu, 1e-2)
+    oc.step()
+    og.step()
+    for o, ps in ((oc, cpu), (og, gpu)):       # groups added later carry every key, as torch requires
+        o.add_param_group(dict(params=[ps[1]], use_muon=True, lr=0.05, momentum=0.9, weight_decay=0.0))
+        o.add_param_group(dict(params=[ps[2]], use_muon=False, lr=1e-3, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.0))
+    for step in range(2):
+        _set_grads(cpu, gpu, 1e-2)
+        oc.step()
+        og.step()
+    for pc, pg in zip(cpu[:2], gpu[:2]):
+        assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 3e-3, tuple(pc.shape)
+    np.testing.assert_allclose(gpu[2].detach().cpu().numpy(), cpu[2].detach().numpy(), rtol=TOL_ADAM, atol=1e-8)
+    assert og.state[gpu[2]]["step"] == 2 and og.state[gpu[1]]["momentum_buffer"].shape == (48, 48)
+
+
+def test_checkpoint_in_the_reference_state_layout(M):
+    """A state dict with the keys the reference writes (muon.py:95-96, 250-254: momentum_buffer;
+    exp_avg, exp_avg_sq, step as a Python int; group keys of muon.py:207-222) loads into both
+    implementations and they keep stepping alike; the state dict written afterwards has the same
+    layout."""
+    cpu, gpu = _clone_params([(72, 40), (10, 24)], 0.02, 1304)
+    torch.manual_seed(1305)
+    mom, ea, eas = torch.randn(72, 40) * 1e-2, torch.randn(10, 24) * 1e-2, torch.rand(10, 24) * 1e-4
+    sd = {"state": {0: {"momentum_buffer": mom}, 1: {"exp_avg": ea, "exp_avg_sq": eas, "step": 7}},
+          "param_groups": [
+              {"lr": 0.03, "momentum": 0.9, "weight_decay": 0.02, "use_muon": True, "params": [0]},
+              {"lr": 1e-3, "betas": (0.8, 0.9), "eps": 1e-8, "weight_decay": 0.1, "use_muon": False, "params": [1]}]}
+    mk = lambda cls, ps: cls([dict(params=[ps[0]], use_muon=True), dict(params=[ps[1]], use_muon=False)])
+    oc, og = mk(O.OracleSingleDeviceMuonWithAuxAdam, cpu), mk(M.SingleDeviceMuonWithAuxAdam, gpu)
+    oc.load_state_dict(copy.deepcopy(sd))
+    og.load_state_dict(copy.deepcopy(sd))
+    assert og.state[gpu[0]]["momentum_buffer"].is_cuda and og.param_groups[0]["momentum"] == 0.9
+    for step in range(2):
+        _set_grads(cpu, gpu, 1e-2)
+        oc.step()
+        og.step()
+    assert O.rel_fro(gpu[0].detach().cpu(), cpu[0].detach()) <= 3e-3
+    np.testing.assert_allclose(gpu[1].detach().cpu().numpy(), cpu[1].detach().numpy(), rtol=TOL_ADAM, atol=1e-8)
+    out = og.state_dict()
+    assert set(out["state"][0].keys()) == {"momentum_buffer"}
+    assert set(out["state"][1].keys()) == {"exp_avg", "exp_avg_sq", "step"} and out["state"][1]["step"] == 9
+    assert out["param_groups"][1]["betas"] == (0.8, 0.9) and out["param_groups"][0]["use_muon"] is True
+    np.testing.assert_allclose(out["state"][0]["momentum_buffer"].cpu().numpy(),
+                               oc.state_dict()["state"][0]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-10)
