@@ -37,7 +37,10 @@ extern "C" {
                                        reference's bf16 tensor expression does (muon.py:282-287) */
 #define MUON_AMD_ROUND_FUSED     0  /* one bf16 rounding per stored output (closer to fp32) */
 
-/* Source dtype of MuonMatDesc.grad. */
+/* Storage type of the caller's tensors of one matrix / Adam tensor: gradient, optimizer state and
+ * parameter share it, as they do in the reference (state is zeros_like(p), muon.py:95-96,
+ * 250-252).  Arithmetic is fp32 either way; with bf16 storage every tensor expression of the
+ * reference rounds to bf16, and so do the kernels. */
 #define MUON_AMD_SRC_F32   0
 #define MUON_AMD_SRC_BF16  1
 
@@ -57,9 +60,9 @@ extern "C" {
  * indexing instead of a pass of its own.
  * ------------------------------------------------------------------------------------------ */
 typedef struct MuonMatDesc {
-    void*     grad;        /* rows*cols, fp32 (or bf16 per src_dtype): gradient / NS input    */
-    float*    momentum;    /* rows*cols fp32 momentum buffer, or NULL (plain NS)              */
-    float*    param;       /* rows*cols fp32 parameter, or NULL                               */
+    void*     grad;        /* rows*cols of src_dtype: gradient / NS input                     */
+    void*     momentum;    /* rows*cols of src_dtype: momentum buffer, or NULL (plain NS)     */
+    void*     param;       /* rows*cols of src_dtype: parameter, or NULL                      */
     uint16_t* out;         /* rows*cols bf16 functional output, or NULL                       */
     uint16_t* u;           /* rows*cols bf16 scratch: update before normalisation             */
     uint16_t* direct;      /* rows_p x cols_p bf16 normalised matrix, parameter orientation   */
@@ -71,7 +74,7 @@ typedef struct MuonMatDesc {
     int32_t   rows_p, cols_p;
     int32_t   ld_direct;   /* leading dimension (elements) of direct and result, >= cols_p    */
     int32_t   ld_transp;   /* leading dimension (elements) of transp, >= rows_p               */
-    int32_t   src_dtype;   /* MUON_AMD_SRC_*                                                  */
+    int32_t   src_dtype;   /* MUON_AMD_SRC_*: storage type of grad, momentum and param        */
     float     scale;       /* max(1, grad.size(-2)/grad.size(-1))**0.5  (muon.py:14)          */
     int32_t   part_begin;  /* first global block id of this matrix in the momentum launch     */
     int32_t   part_end;    /* one past the last                                               */
@@ -105,12 +108,14 @@ typedef struct MuonTileJob {
 
 /* One tensor of the auxiliary Adam group. */
 typedef struct MuonAdamDesc {
-    float* param;        /* numel fp32, or NULL when `update` is used instead                 */
-    const float* grad;   /* numel fp32                                                        */
-    float* exp_avg;      /* numel fp32                                                        */
-    float* exp_avg_sq;   /* numel fp32                                                        */
-    float* update;       /* numel fp32 functional output (adam_update's return), or NULL      */
+    void* param;         /* numel of dtype, or NULL when `update` is used instead             */
+    const void* grad;    /* numel of dtype                                                    */
+    void* exp_avg;       /* numel of dtype                                                    */
+    void* exp_avg_sq;    /* numel of dtype                                                    */
+    void* update;        /* numel of dtype: functional output (adam_update's return), or NULL */
     int64_t numel;
+    int32_t dtype;       /* MUON_AMD_SRC_*: storage type of all five tensors                  */
+    int32_t reserved;    /* 0                                                                 */
 } MuonAdamDesc;
 
 int         muon_amd_abi_version(void);

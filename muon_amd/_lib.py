@@ -35,7 +35,7 @@ GEMM_DESC = np.dtype(
 TILE_JOB = np.dtype([("desc", "<i4"), ("i0", "<i4"), ("j0", "<i4"), ("diag", "<i4")], align=True)
 ADAM_DESC = np.dtype(
     [("param", "<u8"), ("grad", "<u8"), ("exp_avg", "<u8"), ("exp_avg_sq", "<u8"),
-     ("update", "<u8"), ("numel", "<i8")],
+     ("update", "<u8"), ("numel", "<i8"), ("dtype", "<i4"), ("reserved", "<i4")],
     align=True)
 
 _c_int = ctypes.c_int

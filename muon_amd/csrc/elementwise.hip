@@ -60,6 +60,39 @@ __device__ __forceinline__ bool aligned_to(const void* p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }
 
+// Storage type of gradients, optimizer state and parameters: fp32, or bf16 (a model kept in
+// bf16).  Arithmetic is fp32 either way, as torch's kernels do for bf16 tensors; `rnd` is where
+// a value the reference holds in a tensor of the storage type gets that tensor's rounding.
+template <typename T>
+struct Stored;
+template <>
+struct Stored<float> {
+    static constexpr uintptr_t kAlign = 16;                 // of a 4-element access
+    static __device__ __forceinline__ f32x4 ld4(const float* p) { return gld4(p); }
+    static __device__ __forceinline__ void st4(float* p, f32x4 v) { gst4(p, v); }
+    static __device__ __forceinline__ float ld(const float* p) { return *p; }
+    static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+    static __device__ __forceinline__ float rnd(float v) { return v; }
+};
+template <>
+struct Stored<uint16_t> {
+    static constexpr uintptr_t kAlign = 8;
+    static __device__ __forceinline__ f32x4 ld4(const uint16_t* p) {
+        const u32x2e r = gld2u(p);
+        return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+    }
+    static __device__ __forceinline__ void st4(uint16_t* p, f32x4 v) {
+        u32x2e pk;
+        pk.x = pack2bf(v[0], v[1]);
+        pk.y = pack2bf(v[2], v[3]);
+        gst2u(p, pk);
+    }
+    static __device__ __forceinline__ float ld(const uint16_t* p) { return bf2f(*p); }
+    static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = f2bf(v); }
+    static __device__ __forceinline__ float rnd(float v) { return round_bf(v); }
+};
+
 // Sum of `v` over a 256-thread block, valid in thread 0.
 __device__ __forceinline__ float block_sum_256(float v, float* smem4) {
     v = wave_sum(v);
@@ -72,45 +105,41 @@ __device__ __forceinline__ float block_sum_256(float v, float* smem4) {
 // ------------------------------------------------------------------------------------------
 // momentum: muon.py:9-10 + the bf16 cast of muon.py:277 + partial sums for muon.py:282
 // ------------------------------------------------------------------------------------------
+template <typename T>
 __device__ __forceinline__ float momentum_one(float g, float* m_io, bool has_m, float w,
                                               float beta, int nesterov, float* g_out) {
     if (!has_m) return g;
-    const float m_new = lerp_torch(*m_io, g, w);          // momentum.lerp_(grad, 1 - beta)
+    const float m_new = Stored<T>::rnd(lerp_torch(*m_io, g, w));      // momentum.lerp_(grad, 1 - beta)
     *m_io = m_new;
     if (!nesterov) return m_new;
-    const float u = lerp_torch(g, m_new, beta);           // grad.lerp_(momentum, beta)
+    const float u = Stored<T>::rnd(lerp_torch(g, m_new, beta));       // grad.lerp_(momentum, beta)
     *g_out = u;
     return u;
 }
 
-__global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
-    const MuonMatDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, float w,
-    float beta, int nesterov, int mutate_grad) {
-    __shared__ float red[4];
-    const int b = blockIdx.x;
-    const int mi = find_segment(prefix, nmat, b);
-    const MuonMatDesc d = descs[mi];
+// One block's share of a matrix whose gradient and momentum are stored as T.
+template <typename T>
+__device__ __forceinline__ float momentum_block(const MuonMatDesc& d, int64_t block_base, float w,
+                                                float beta, int nesterov, int mutate_grad) {
     const int64_t numel = static_cast<int64_t>(d.rows) * d.cols;
-    const int64_t block_base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
     const bool has_m = d.momentum != nullptr;
     const bool write_g = has_m && nesterov && mutate_grad;
-    const bool src_bf16 = d.src_dtype == MUON_AMD_SRC_BF16;
-    float* __restrict__ mom = d.momentum;
+    T* __restrict__ g = static_cast<T*>(d.grad);
+    T* __restrict__ mom = static_cast<T*>(d.momentum);
     uint16_t* __restrict__ u = d.u;
     float ss = 0.f;
-    const bool aligned = !src_bf16 && aligned_to(d.grad, 16) && aligned_to(mom, 16) && aligned_to(u, 8);
+    const bool aligned = aligned_to(g, Stored<T>::kAlign) && aligned_to(mom, Stored<T>::kAlign) && aligned_to(u, 8);
 
     for (int pass = 0; pass < EW_PASSES; ++pass) {
         const int64_t base = block_base + static_cast<int64_t>(pass) * EW_PASS_ELEMS;
         if (base >= numel) break;
         if (aligned && base + EW_PASS_ELEMS <= numel) {
-            float* __restrict__ g = static_cast<float*>(d.grad);
             f32x4 gv[EW_ITERS], mv[EW_ITERS];
 #pragma unroll
             for (int it = 0; it < EW_ITERS; ++it) {
                 const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
-                gv[it] = gld4(g + e);
-                if (has_m) mv[it] = gld4(mom + e);
+                gv[it] = Stored<T>::ld4(g + e);
+                if (has_m) mv[it] = Stored<T>::ld4(mom + e);
                 else mv[it] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
@@ -121,14 +150,14 @@ __global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     float gout = gg[k], mk = mm[k];
-                    uu[k] = momentum_one(gg[k], &mk, has_m, w, beta, nesterov, &gout);
+                    uu[k] = momentum_one<T>(gg[k], &mk, has_m, w, beta, nesterov, &gout);
                     mm[k] = mk;
                     gg[k] = gout;
                     const float ub = round_bf(uu[k]);
                     ss = fmaf(ub, ub, ss);
                 }
-                if (has_m) gst4(mom + e, mm);
-                if (write_g) gst4(g + e, gg);
+                if (has_m) Stored<T>::st4(mom + e, mm);
+                if (write_g) Stored<T>::st4(g + e, gg);
                 u32x2e pk;
                 pk.x = pack2bf(uu[0], uu[1]);
                 pk.y = pack2bf(uu[2], uu[3]);
@@ -141,13 +170,12 @@ __global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
                 for (int k = 0; k < EW_VEC; ++k) {
                     const int64_t e = e0 + k;
                     if (e >= numel) break;
-                    float gval = src_bf16 ? bf2f(static_cast<const uint16_t*>(d.grad)[e])
-                                          : static_cast<const float*>(d.grad)[e];
-                    float mval = has_m ? mom[e] : 0.f;
+                    const float gval = Stored<T>::ld(g + e);
+                    float mval = has_m ? Stored<T>::ld(mom + e) : 0.f;
                     float gout = gval;
-                    const float uval = momentum_one(gval, &mval, has_m, w, beta, nesterov, &gout);
-                    if (has_m) mom[e] = mval;
-                    if (write_g) static_cast<float*>(d.grad)[e] = gout;
+                    const float uval = momentum_one<T>(gval, &mval, has_m, w, beta, nesterov, &gout);
+                    if (has_m) Stored<T>::st(mom + e, mval);
+                    if (write_g) Stored<T>::st(g + e, gout);
                     const uint16_t ub = f2bf(uval);
                     u[e] = ub;
                     const float uf = bf2f(ub);
@@ -156,6 +184,20 @@ __global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
             }
         }
     }
+    return ss;
+}
+
+__global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
+    const MuonMatDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, float w,
+    float beta, int nesterov, int mutate_grad) {
+    __shared__ float red[4];
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonMatDesc d = descs[mi];
+    const int64_t block_base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
+    const float ss = d.src_dtype == MUON_AMD_SRC_BF16
+                         ? momentum_block<uint16_t>(d, block_base, w, beta, nesterov, mutate_grad)
+                         : momentum_block<float>(d, block_base, w, beta, nesterov, mutate_grad);
     const float total = block_sum_256(ss, red);
     if (threadIdx.x == 0) d.partials[b] = total;
 }
@@ -255,19 +297,22 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
 // ------------------------------------------------------------------------------------------
 // apply: muon.py:14 (aspect scale, in bf16), muon.py:98-99 (decoupled decay + step)
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __restrict__ descs,
-                                                            const int32_t* __restrict__ prefix,
-                                                            int nmat, float neg_lr, float wd_factor) {
-    const int b = blockIdx.x;
-    const int mi = find_segment(prefix, nmat, b);
-    const MuonMatDesc d = descs[mi];
+// p.mul_(1 - lr*wd); p.add_(update, alpha=-lr): two tensor operations in the reference, so a
+// parameter stored as bf16 is rounded after each (for fp32 storage rnd is the identity).
+template <typename T>
+__device__ __forceinline__ float apply_one(float p, float us, float neg_lr, float wd_factor) {
+    return Stored<T>::rnd(fmaf(neg_lr, us, Stored<T>::rnd(p * wd_factor)));
+}
+
+template <typename T>
+__device__ __forceinline__ void apply_block(const MuonMatDesc& d, int64_t block_base, float neg_lr,
+                                            float wd_factor) {
     const int64_t numel = static_cast<int64_t>(d.rows) * d.cols;
-    const int64_t block_base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
-    float* __restrict__ p = d.param;
+    T* __restrict__ p = static_cast<T*>(d.param);
     uint16_t* __restrict__ out = d.out;
     const uint16_t* __restrict__ res = d.result;
     const float scale = d.scale;
-    const bool aligned = (d.cols % 4 == 0) && aligned_to(p, 16) && aligned_to(out, 8);
+    const bool aligned = (d.cols % 4 == 0) && aligned_to(p, Stored<T>::kAlign) && aligned_to(out, 8);
     for (int pass = 0; pass < EW_PASSES; ++pass) {
         const int64_t base = block_base + static_cast<int64_t>(pass) * EW_PASS_ELEMS;
         if (base >= numel) break;
@@ -279,7 +324,7 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
                 const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
                 const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
                 ov[it] = gld2u(res + static_cast<int64_t>(rr) * d.ld_direct + cc);
-                if (p) pv[it] = gld4(p + e);
+                if (p) pv[it] = Stored<T>::ld4(p + e);
                 else pv[it] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
@@ -292,9 +337,9 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     us[k] = round_bf(o[k] * scale);
-                    pp[k] = fmaf(neg_lr, us[k], pp[k] * wd_factor);
+                    pp[k] = apply_one<T>(pp[k], us[k], neg_lr, wd_factor);
                 }
-                if (p) gst4(p + e, pp);
+                if (p) Stored<T>::st4(p + e, pp);
                 if (out) {
                     u32x2e pk;
                     pk.x = pack2bf(us[0], us[1]);
@@ -311,7 +356,7 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
                     if (e >= numel) break;
                     const int rr = static_cast<int>(e / d.cols), cc = static_cast<int>(e - static_cast<int64_t>(rr) * d.cols);
                     const float us = round_bf(bf2f(res[static_cast<int64_t>(rr) * d.ld_direct + cc]) * scale);
-                    if (p) p[e] = fmaf(neg_lr, us, p[e] * wd_factor);
+                    if (p) Stored<T>::st(p + e, apply_one<T>(Stored<T>::ld(p + e), us, neg_lr, wd_factor));
                     if (out) out[e] = f2bf(us);
                 }
             }
@@ -319,16 +364,95 @@ __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __
     }
 }
 
+__global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __restrict__ descs,
+                                                            const int32_t* __restrict__ prefix,
+                                                            int nmat, float neg_lr, float wd_factor) {
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonMatDesc d = descs[mi];
+    const int64_t block_base = static_cast<int64_t>(b - prefix[mi]) * EW_BLOCK_ELEMS;
+    if (d.src_dtype == MUON_AMD_SRC_BF16) apply_block<uint16_t>(d, block_base, neg_lr, wd_factor);
+    else apply_block<float>(d, block_base, neg_lr, wd_factor);
+}
+
 // ------------------------------------------------------------------------------------------
 // auxiliary Adam: muon.py:104-109 + 257-258
 // ------------------------------------------------------------------------------------------
+// Every tensor expression of muon.py:105-109 leaves a tensor of the storage type, so for bf16
+// storage each of them rounds (grad.square(), both lerps, both bias corrections, the square root,
+// "+ eps", the quotient); for fp32 storage rnd is the identity.
+template <typename T>
 __device__ __forceinline__ float adam_one(float g, float* m, float* v, float w1, float w2,
                                           float eps, float bias1, float bias2) {
-    *m = lerp_torch(*m, g, w1);
-    *v = lerp_torch(*v, g * g, w2);
-    const float mc = *m / bias1;
-    const float vc = *v / bias2;
-    return mc / (sqrtf(vc) + eps);
+    typedef Stored<T> S;
+    *m = S::rnd(lerp_torch(*m, g, w1));
+    *v = S::rnd(lerp_torch(*v, S::rnd(g * g), w2));
+    const float mc = S::rnd(*m / bias1);
+    const float vc = S::rnd(*v / bias2);
+    return S::rnd(mc / S::rnd(S::rnd(sqrtf(vc)) + eps));
+}
+
+template <typename T>
+__device__ __forceinline__ void adam_block(const MuonAdamDesc& d, int64_t block_base, float neg_lr,
+                                           float wd_factor, float w1, float w2, float eps,
+                                           float bias1, float bias2) {
+    const int64_t numel = d.numel;
+    T* __restrict__ p = static_cast<T*>(d.param);
+    const T* __restrict__ g = static_cast<const T*>(d.grad);
+    T* __restrict__ m = static_cast<T*>(d.exp_avg);
+    T* __restrict__ v = static_cast<T*>(d.exp_avg_sq);
+    T* __restrict__ upd = static_cast<T*>(d.update);
+    constexpr uintptr_t A = Stored<T>::kAlign;
+    const bool aligned = aligned_to(p, A) && aligned_to(g, A) && aligned_to(m, A) && aligned_to(v, A) &&
+                         aligned_to(upd, A);
+    for (int pass = 0; pass < EW_PASSES; ++pass) {
+        const int64_t base = block_base + static_cast<int64_t>(pass) * EW_PASS_ELEMS;
+        if (base >= numel) break;
+        if (aligned && base + EW_PASS_ELEMS <= numel) {
+            f32x4 gv[EW_ITERS], mv[EW_ITERS], vv[EW_ITERS], pv[EW_ITERS];
+#pragma unroll
+            for (int it = 0; it < EW_ITERS; ++it) {
+                const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+                gv[it] = Stored<T>::ld4(g + e);
+                mv[it] = Stored<T>::ld4(m + e);
+                vv[it] = Stored<T>::ld4(v + e);
+                if (p) pv[it] = Stored<T>::ld4(p + e);
+                else pv[it] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int it = 0; it < EW_ITERS; ++it) {
+                const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+                f32x4 mm = mv[it], v2 = vv[it], pp = pv[it], uu;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float mk = mm[k], vk = v2[k];
+                    uu[k] = adam_one<T>(gv[it][k], &mk, &vk, w1, w2, eps, bias1, bias2);
+                    mm[k] = mk;
+                    v2[k] = vk;
+                    pp[k] = apply_one<T>(pp[k], uu[k], neg_lr, wd_factor);
+                }
+                Stored<T>::st4(m + e, mm);
+                Stored<T>::st4(v + e, v2);
+                if (p) Stored<T>::st4(p + e, pp);
+                if (upd) Stored<T>::st4(upd + e, uu);
+            }
+        } else {
+            for (int it = 0; it < EW_ITERS; ++it) {
+                const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+#pragma unroll
+                for (int k = 0; k < EW_VEC; ++k) {
+                    const int64_t e = e0 + k;
+                    if (e >= numel) break;
+                    float mm = Stored<T>::ld(m + e), v2 = Stored<T>::ld(v + e);
+                    const float uu = adam_one<T>(Stored<T>::ld(g + e), &mm, &v2, w1, w2, eps, bias1, bias2);
+                    Stored<T>::st(m + e, mm);
+                    Stored<T>::st(v + e, v2);
+                    if (p) Stored<T>::st(p + e, apply_one<T>(Stored<T>::ld(p + e), uu, neg_lr, wd_factor));
+                    if (upd) Stored<T>::st(upd + e, uu);
+                }
+            }
+        }
+    }
 }
 
 __global__ __launch_bounds__(EW_THREADS) void adam_kernel(const MuonAdamDesc* __restrict__ descs,
@@ -339,63 +463,11 @@ __global__ __launch_bounds__(EW_THREADS) void adam_kernel(const MuonAdamDesc* __
     const int b = blockIdx.x;
     const int ti = find_segment(prefix, ntensors, b);
     const MuonAdamDesc d = descs[ti];
-    const int64_t numel = d.numel;
     const int64_t block_base = static_cast<int64_t>(b - prefix[ti]) * EW_BLOCK_ELEMS;
-    float* __restrict__ p = d.param;
-    const float* __restrict__ g = d.grad;
-    float* __restrict__ m = d.exp_avg;
-    float* __restrict__ v = d.exp_avg_sq;
-    float* __restrict__ upd = d.update;
-    const bool aligned = aligned_to(p, 16) && aligned_to(g, 16) && aligned_to(m, 16) && aligned_to(v, 16) &&
-                         aligned_to(upd, 16);
-    for (int pass = 0; pass < EW_PASSES; ++pass) {
-        const int64_t base = block_base + static_cast<int64_t>(pass) * EW_PASS_ELEMS;
-        if (base >= numel) break;
-        if (aligned && base + EW_PASS_ELEMS <= numel) {
-            f32x4 gv[EW_ITERS], mv[EW_ITERS], vv[EW_ITERS], pv[EW_ITERS];
-#pragma unroll
-            for (int it = 0; it < EW_ITERS; ++it) {
-                const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
-                gv[it] = gld4(g + e);
-                mv[it] = gld4(m + e);
-                vv[it] = gld4(v + e);
-                if (p) pv[it] = gld4(p + e);
-                else pv[it] = f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-#pragma unroll
-            for (int it = 0; it < EW_ITERS; ++it) {
-                const int64_t e = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
-                f32x4 mm = mv[it], v2 = vv[it], pp = pv[it], uu;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    float mk = mm[k], vk = v2[k];
-                    uu[k] = adam_one(gv[it][k], &mk, &vk, w1, w2, eps, bias1, bias2);
-                    mm[k] = mk;
-                    v2[k] = vk;
-                    pp[k] = fmaf(neg_lr, uu[k], pp[k] * wd_factor);
-                }
-                gst4(m + e, mm);
-                gst4(v + e, v2);
-                if (p) gst4(p + e, pp);
-                if (upd) gst4(upd + e, uu);
-            }
-        } else {
-            for (int it = 0; it < EW_ITERS; ++it) {
-                const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
-#pragma unroll
-                for (int k = 0; k < EW_VEC; ++k) {
-                    const int64_t e = e0 + k;
-                    if (e >= numel) break;
-                    float mm = m[e], v2 = v[e];
-                    const float uu = adam_one(g[e], &mm, &v2, w1, w2, eps, bias1, bias2);
-                    m[e] = mm;
-                    v[e] = v2;
-                    if (p) p[e] = fmaf(neg_lr, uu, p[e] * wd_factor);
-                    if (upd) upd[e] = uu;
-                }
-            }
-        }
-    }
+    if (d.dtype == MUON_AMD_SRC_BF16)
+        adam_block<uint16_t>(d, block_base, neg_lr, wd_factor, w1, w2, eps, bias1, bias2);
+    else
+        adam_block<float>(d, block_base, neg_lr, wd_factor, w1, w2, eps, bias1, bias2);
 }
 
 }  // namespace muon_amd
@@ -429,8 +501,6 @@ int muon_amd_validate_mats(const MuonMatDesc* descs, int nmat, const int32_t* bl
         MUON_REQUIRE(d.param || d.out, "mat %d: neither param nor out given", i);
         MUON_REQUIRE(d.src_dtype == MUON_AMD_SRC_F32 || d.src_dtype == MUON_AMD_SRC_BF16,
                      "mat %d: src_dtype=%d", i, d.src_dtype);
-        MUON_REQUIRE(d.src_dtype == MUON_AMD_SRC_F32 || d.momentum == nullptr,
-                     "mat %d: momentum needs an fp32 gradient", i);
         MUON_REQUIRE((reinterpret_cast<uintptr_t>(d.direct) % 16) == 0 &&
                          (reinterpret_cast<uintptr_t>(d.transp) % 16) == 0 &&
                          (reinterpret_cast<uintptr_t>(d.result) % 16) == 0 &&

@@ -99,6 +99,7 @@ class _ChunkRuntime:
                    "validate_mats")
         self.mat_dev = _upload(d, self.device)
         self.mat_key = key
+        self.src_dtypes = list(src_dtypes)
 
     def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor):
         lib = _lib.load()
@@ -108,7 +109,12 @@ class _ChunkRuntime:
         mats = self.mat_dev.data_ptr()
         elts = sum(lay.numel for lay in c.layouts)
         padded = sum(lay.mp * lay.np_ for lay in c.layouts)
-        _launch("momentum", elts * 14, lambda: _lib.check(lib.muon_amd_momentum(
+        # algorithmic bytes: gradient, momentum (read + write) and parameter (read + write) in
+        # their storage type, the bf16 update written once and read once
+        store = [2 if t == _lib.SRC_BF16 else 4 for t in self.src_dtypes]
+        mom_bytes = sum(lay.numel * (3 * sz + 2) for lay, sz in zip(c.layouts, store))
+        apply_bytes = sum(lay.numel * (2 * sz + 2) for lay, sz in zip(c.layouts, store))
+        _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
             int(mutate_grad), s), "momentum"))
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
@@ -131,7 +137,7 @@ class _ChunkRuntime:
             _launch("ns_gemm/update", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm(
                 self.gemm_ptr[ph], self.full_jobs_ptr, len(c.full_jobs), c.tile_class, al, be, ga,
                 flags, s), "ns_gemm"))
-        _launch("apply", elts * 10, lambda: _lib.check(lib.muon_amd_apply(
+        _launch("apply", apply_bytes, lambda: _lib.check(lib.muon_amd_apply(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply"))
 
 
@@ -179,8 +185,10 @@ class AdamGroupEngine:
         self.desc_dev = None
         self.key = None
 
-    def run(self, params, grads, exp_avgs, exp_avg_sqs, updates, *, lr, weight_decay, betas, eps, step):
-        key = (tuple(params), tuple(grads), tuple(exp_avgs), tuple(exp_avg_sqs), tuple(updates))
+    def run(self, params, grads, exp_avgs, exp_avg_sqs, updates, *, lr, weight_decay, betas, eps, step,
+            dtypes=None):
+        dtypes = [_lib.SRC_F32] * len(self.numels) if dtypes is None else list(dtypes)
+        key = (tuple(params), tuple(grads), tuple(exp_avgs), tuple(exp_avg_sqs), tuple(updates), tuple(dtypes))
         if key != self.key:
             d = np.zeros(len(self.numels), dtype=_lib.ADAM_DESC)
             d["param"] = params
@@ -189,6 +197,7 @@ class AdamGroupEngine:
             d["exp_avg_sq"] = exp_avg_sqs
             d["update"] = updates
             d["numel"] = self.numels
+            d["dtype"] = dtypes
             self.desc_dev = _upload(d, self.device)
             self.key = key
         lib = _lib.load()
@@ -196,6 +205,7 @@ class AdamGroupEngine:
         w2 = 1 - betas[1]
         bias1 = 1 - betas[0] ** step
         bias2 = 1 - betas[1] ** step
-        _launch("adam", sum(self.numels) * 28, lambda: _lib.check(lib.muon_amd_adam(
+        nbytes = sum(n * (14 if t == _lib.SRC_BF16 else 28) for n, t in zip(self.numels, dtypes))
+        _launch("adam", nbytes, lambda: _lib.check(lib.muon_amd_adam(
             self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels), self.nblocks, lr,
             1 - lr * weight_decay, w1, w2, eps, bias1, bias2, _stream_ptr(self.device)), "adam"))

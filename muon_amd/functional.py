@@ -83,8 +83,8 @@ def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
     require_gpu_tensor(grad, "grad")
     require_gpu_tensor(momentum, "momentum")
     assert grad.ndim >= 2                                  # muon.py:275 via muon.py:13
-    if grad.dtype != torch.float32 or momentum.dtype != torch.float32:
-        raise TypeError("muon_update needs fp32 grad and momentum")
+    if grad.dtype != momentum.dtype or grad.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError("muon_update needs grad and momentum of one dtype, fp32 or bf16")
     if not (grad.is_contiguous() and momentum.is_contiguous()):
         raise ValueError("muon_update needs contiguous grad and momentum (they are updated in place)")
     assert grad.shape == momentum.shape
@@ -102,22 +102,22 @@ def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
     with torch.cuda.device(grad.device):
         eng = _cached(("ns", grad.device, rows, cols, batch, int(ns_steps), ref),
                       lambda: MuonGroupEngine([(rows, cols)] * batch, grad.device, int(ns_steps), ref))
-        gsz, osz = rows * cols * 4, rows * cols * 2
+        gsz, osz = rows * cols * grad.element_size(), rows * cols * 2
         eng.run([grad.data_ptr() + b * gsz for b in range(batch)],
                 [momentum.data_ptr() + b * gsz for b in range(batch)], [0] * batch,
                 [out.data_ptr() + b * osz for b in range(batch)], [scale] * batch,
-                [_lib.SRC_F32] * batch, beta=beta, nesterov=bool(nesterov), mutate_grad=True,
+                [_src_dtype(grad)] * batch, beta=beta, nesterov=bool(nesterov), mutate_grad=True,
                 eps=1e-7, lr=0.0, weight_decay=0.0)
     return out
 
 
 def adam_update(grad, buf1, buf2, step, betas, eps) -> torch.Tensor:
     """Reference muon.py:104-109: updates both moment buffers in place and returns the
-    bias-corrected Adam direction (fp32)."""
+    bias-corrected Adam direction (in the dtype of the inputs: fp32 or bf16)."""
     for name, t in (("grad", grad), ("buf1", buf1), ("buf2", buf2)):
         require_gpu_tensor(t, name)
-        if t.dtype != torch.float32:
-            raise TypeError("adam_update needs fp32 tensors")
+        if t.dtype != grad.dtype or t.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError("adam_update needs tensors of one dtype, fp32 or bf16")
     if not (buf1.is_contiguous() and buf2.is_contiguous()):
         raise ValueError("adam_update needs contiguous moment buffers (they are updated in place)")
     grad = grad.contiguous()
@@ -127,5 +127,5 @@ def adam_update(grad, buf1, buf2, step, betas, eps) -> torch.Tensor:
     with torch.cuda.device(grad.device):
         eng = _cached(("adam", grad.device, grad.numel()), lambda: AdamGroupEngine([grad.numel()], grad.device))
         eng.run([0], [grad.data_ptr()], [buf1.data_ptr()], [buf2.data_ptr()], [out.data_ptr()],
-                lr=0.0, weight_decay=0.0, betas=betas, eps=float(eps), step=step)
+                lr=0.0, weight_decay=0.0, betas=betas, eps=float(eps), step=step, dtypes=[_src_dtype(grad)])
     return out

@@ -9,9 +9,8 @@ from __future__ import annotations
 
 import torch
 
-from . import _lib
 from .engine import AdamGroupEngine, MuonGroupEngine, require_gpu_tensor
-from .functional import _rounding_flag
+from .functional import _rounding_flag, _src_dtype
 
 NS_STEPS = 5          # the reference classes never pass a step count: muon_update's default rules
 NESTEROV = True       # likewise (muon.py:8)
@@ -42,16 +41,16 @@ class _MuonBase(torch.optim.Optimizer):
     @staticmethod
     def _check_param(p):
         require_gpu_tensor(p, "parameter")
-        if p.dtype != torch.float32:
-            raise NotImplementedError(f"muon_amd updates fp32 parameters; got {p.dtype}")
+        if p.dtype not in (torch.float32, torch.bfloat16):
+            raise NotImplementedError(f"muon_amd updates fp32 and bf16 parameters; got {p.dtype}")
 
     @staticmethod
     def _grad_of(p):
         if p.grad is None:
             p.grad = torch.zeros_like(p)          # muon.py:91-93 "Force synchronization"
         g = p.grad
-        if g.dtype != torch.float32 or g.is_sparse:
-            raise NotImplementedError("muon_amd needs dense fp32 gradients")
+        if g.dtype != p.dtype or g.is_sparse:
+            raise NotImplementedError("muon_amd needs dense gradients of the parameter's dtype")
         return g
 
     @staticmethod
@@ -69,15 +68,15 @@ class _MuonBase(torch.optim.Optimizer):
     @staticmethod
     def _state_tensor(state, key, p):
         t = state[key]
-        if t.dtype != torch.float32 or t.device != p.device or t.shape != p.shape:
-            raise NotImplementedError(f"{key} must be an fp32 tensor of the parameter's shape on its device")
+        if t.dtype != p.dtype or t.device != p.device or t.shape != p.shape:
+            raise NotImplementedError(f"{key} must be a tensor of the parameter's dtype and shape on its device")
         return t
 
     def _muon_group_step(self, gi, group):
         params = [p for p in group["params"] if p.numel() > 0]
         if not params:
             return
-        grads, moms, ptrs, shapes, scales, writebacks, keep = [], [], [], [], [], [], []
+        grads, moms, ptrs, shapes, scales, dtypes, writebacks, keep = [], [], [], [], [], [], [], []
         for p in params:
             self._check_param(p)
             assert p.ndim >= 2                    # muon.py:275 (reached through muon.py:13)
@@ -96,9 +95,10 @@ class _MuonBase(torch.optim.Optimizer):
                 batch = p.numel() // (rows * cols)
             scale = max(1, p.size(-2) / p.size(-1)) ** 0.5             # muon.py:14
             for k in range(batch):
-                off = k * rows * cols * 4
+                off = k * rows * cols * p.element_size()
                 shapes.append((rows, cols))
                 scales.append(scale)
+                dtypes.append(_src_dtype(p))
                 grads.append(g.data_ptr() + off)
                 moms.append(m.data_ptr() + off)
                 ptrs.append(pc.data_ptr() + off)
@@ -111,7 +111,7 @@ class _MuonBase(torch.optim.Optimizer):
             self._muon_engines[key] = eng
         n = len(shapes)
         with torch.cuda.device(device):
-            eng.run(grads, moms, ptrs, [0] * n, scales, [_lib.SRC_F32] * n,
+            eng.run(grads, moms, ptrs, [0] * n, scales, dtypes,
                     beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad,
                     eps=1e-7, lr=group["lr"], weight_decay=group["weight_decay"])
             for dst, src in writebacks:           # stream ordered after the launches
@@ -145,7 +145,7 @@ class _MuonBase(torch.optim.Optimizer):
                         [t[2].data_ptr() for _, t in items], [t[3].data_ptr() for _, t in items],
                         [0] * len(items),
                         lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"],
-                        eps=group["eps"], step=step)
+                        eps=group["eps"], step=step, dtypes=[_src_dtype(p) for p, _ in items])
         for dst, src in writebacks:
             dst.copy_(src)
 

@@ -440,3 +440,79 @@ def test_checkpoint_in_the_reference_state_layout(M):
     assert out["param_groups"][1]["betas"] == (0.8, 0.9) and out["param_groups"][0]["use_muon"] is True
     np.testing.assert_allclose(out["state"][0]["momentum_buffer"].cpu().numpy(),
                                oc.state_dict()["state"][0]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-10)
+
+
+# ------------------------------------------------------------------------------------------
+# bf16 storage: parameters, gradients and optimizer state kept in bf16.  The reference then rounds
+# every tensor expression to bf16 (state is zeros_like(p), muon.py:95-96, 250-252); the kernels
+# compute in fp32 and round at the same places.
+# ------------------------------------------------------------------------------------------
+def _ulps_bf16(a, b):
+    """Difference in units of the bf16 spacing at max(|a|, |b|), elementwise (fp32 tensors)."""
+    scale = torch.maximum(a.abs(), b.abs()).clamp_min(1e-30)
+    return (a - b).abs() / (2.0 ** torch.floor(torch.log2(scale)) * 2.0 ** -7)
+
+
+def _assert_bf16_close(got, want, max_flip_fraction, what):
+    got, want = got.detach().float().cpu(), want.detach().float()
+    u = _ulps_bf16(got, want)
+    assert u.max() <= 1.0 + 1e-6, (what, float(u.max()))             # never more than one rounding step
+    assert (u > 0).float().mean() <= max_flip_fraction, (what, float((u > 0).float().mean()))
+
+
+def test_bf16_parameters_step(M):
+    """The oracle's tensor expressions run here on GPU tensors (torch's own kernels, rocBLAS for
+    the bf16 matmuls): for bf16 tensors torch's CPU kernels round the `alpha` of
+    p.add_(update, alpha=-lr) and added Python scalars to bf16 before using them, its GPU kernels
+    keep them in fp32 -- and the reference runs on a GPU (muon.py:98-99, 257-258)."""
+    torch.manual_seed(1310)
+    muon_shapes, adam_shapes = [(256, 384), (96, 64), (3, 40, 24), (16, 8, 3, 3)], [(1000, 64), (33,)]
+    mk_ref = lambda s, std: torch.nn.Parameter(_dev((torch.randn(*s) * std).bfloat16()))
+    ref_m, ref_a = [mk_ref(s, 0.02) for s in muon_shapes], [mk_ref(s, 0.02) for s in adam_shapes]
+    gpu_m = [torch.nn.Parameter(p.detach().clone()) for p in ref_m]
+    gpu_a = [torch.nn.Parameter(p.detach().clone()) for p in ref_a]
+    mk = lambda cls, pm, pa: cls([dict(params=pm, use_muon=True, lr=0.02, weight_decay=0.01),
+                                  dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), weight_decay=0.01)])
+    oc, og = mk(O.OracleSingleDeviceMuonWithAuxAdam, ref_m, ref_a), mk(M.SingleDeviceMuonWithAuxAdam, gpu_m, gpu_a)
+    for step in range(3):
+        for pc, pg in zip(ref_m + ref_a, gpu_m + gpu_a):
+            g = _dev((torch.randn(*pc.shape) * 1e-2).bfloat16())
+            pc.grad, pg.grad = g.clone(), g.clone()
+        oc.step()
+        og.step()
+        for pc, pg in zip(ref_m, gpu_m):
+            assert pg.dtype == torch.bfloat16 and og.state[pg]["momentum_buffer"].dtype == torch.bfloat16
+            # the momentum has no Newton-Schulz in it: same roundings, same bits (bar rare double-rounding ties)
+            _assert_bf16_close(og.state[pg]["momentum_buffer"], oc.state[pc]["momentum_buffer"].cpu(), 1e-3, ("momentum", step))
+            # a parameter is one bf16 rounding of p*(1-lr*wd) - lr*O: the two Newton-Schulz results
+            # differ inside their tolerance, which moves some parameters across a rounding
+            # boundary -- 3e-3 is half a bf16 step in the Frobenius sense
+            assert O.rel_fro(pg.detach().float().cpu(), pc.detach().float().cpu()) <= 3e-3, (tuple(pc.shape), step)
+        for pc, pg in zip(ref_a, gpu_a):
+            _assert_bf16_close(og.state[pg]["exp_avg"], oc.state[pc]["exp_avg"].cpu(), 2e-3, ("exp_avg", step))
+            _assert_bf16_close(og.state[pg]["exp_avg_sq"], oc.state[pc]["exp_avg_sq"].cpu(), 2e-3, ("exp_avg_sq", step))
+            # parameters near zero sit many bf16 steps of their own size away from a neighbour one
+            # step of the update's size off, so the parameter is compared in the Frobenius sense
+            assert (pg.detach().float() != pc.detach().float()).float().mean() <= 5e-3, ("adam param", step)
+            assert O.rel_fro(pg.detach().float().cpu(), pc.detach().float().cpu()) <= 1e-4, ("adam param", step)
+
+
+def test_bf16_functional_updates(M):
+    torch.manual_seed(1311)
+    g = (torch.randn(130, 72) * 1e-2).bfloat16()
+    m = (torch.randn(130, 72) * 1e-2).bfloat16()
+    gc, mc, gg, mg = g.clone(), m.clone(), _dev(g.clone()), _dev(m.clone())
+    want = O.muon_update(gc, mc, beta=0.9, nesterov=True)
+    got = M.muon_update(gg, mg, beta=0.9, nesterov=True)
+    assert got.dtype == torch.bfloat16 and O.rel_fro(got.float().cpu(), want.float()) <= TOL_BF16
+    _assert_bf16_close(mg, mc, 1e-3, "momentum")
+    _assert_bf16_close(gg, gc, 1e-3, "blended grad")        # grad.lerp_ is in place (muon.py:10)
+    b1, b2 = (torch.randn(999) * 1e-2).bfloat16(), (torch.rand(999) * 1e-4).bfloat16()
+    ga = (torch.randn(999) * 1e-2).bfloat16()
+    b1c, b2c, b1g, b2g = b1.clone(), b2.clone(), _dev(b1.clone()), _dev(b2.clone())
+    want = O.adam_update(ga.clone(), b1c, b2c, 3, (0.9, 0.95), 1e-10)
+    got = M.adam_update(_dev(ga.clone()), b1g, b2g, 3, (0.9, 0.95), 1e-10)
+    assert got.dtype == torch.bfloat16
+    _assert_bf16_close(got, want, 5e-3, "adam direction")
+    _assert_bf16_close(b1g, b1c, 2e-3, "exp_avg")
+    _assert_bf16_close(b2g, b2c, 2e-3, "exp_avg_sq")

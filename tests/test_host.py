@@ -39,7 +39,7 @@ def test_struct_layouts_match_the_library():
     assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 120
     assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 88
     assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 16
-    assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 48
+    assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 56
 
 
 def test_entry_points_reject_bad_arguments_without_a_gpu():
