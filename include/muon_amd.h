@@ -36,6 +36,8 @@ extern "C" {
 #define MUON_AMD_ROUND_REFERENCE 1  /* round every intermediate to bf16 exactly where the
                                        reference's bf16 tensor expression does (muon.py:282-287) */
 #define MUON_AMD_ROUND_FUSED     0  /* one bf16 rounding per stored output (closer to fp32) */
+#define MUON_AMD_NORM_UNIT       2  /* muon_amd_norm_finalize only: denom = 1 (no Frobenius
+                                       pre-scale; the AOL variant rescales by rows instead) */
 
 /* Storage type of the caller's tensors of one matrix / Adam tensor: gradient, optimizer state and
  * parameter share it, as they do in the reference (state is zeros_like(p), muon.py:95-96,
@@ -118,6 +120,16 @@ typedef struct MuonAdamDesc {
     int32_t reserved;    /* 0                                                                 */
 } MuonAdamDesc;
 
+/* One matrix of the AOL rescaling step of the 4-iteration variant (muon.py:776-785), in the
+ * wide orientation: X is m_p x n_p with m_p <= n_p (zero padded).                           */
+typedef struct MuonAolDesc {
+    uint16_t* xr;     /* m_p x n_p bf16 (leading dimension ld_n): X, scaled by r along rows     */
+    uint16_t* xc;     /* n_p x m_p bf16 (ld_m): X^T, scaled by r along columns                  */
+    uint16_t* gram;   /* m_p x m_p bf16 (ld_m): A = X X^T, becomes diag(r) A diag(r)            */
+    float*    rvec;   /* m_p floats: r_i = max(sum_j |A_ij|, eps)^-1/2                          */
+    int32_t   m_p, n_p, ld_n, ld_m;
+} MuonAolDesc;
+
 int         muon_amd_abi_version(void);
 const char* muon_amd_last_error(void);
 
@@ -126,6 +138,7 @@ size_t muon_amd_sizeof_mat_desc(void);
 size_t muon_amd_sizeof_gemm_desc(void);
 size_t muon_amd_sizeof_tile_job(void);
 size_t muon_amd_sizeof_adam_desc(void);
+size_t muon_amd_sizeof_aol_desc(void);
 
 /* Elements each block of the flat elementwise launches covers (momentum, apply, adam), and
  * the edge of the square tile of the normalise/transposing launch. */
@@ -179,6 +192,24 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
  * - lr*update (muon.py:98-99); if out: out <- update (what muon_update returns, muon.py:15). */
 int muon_amd_apply(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
                    int nblocks, float lr, float wd_factor, void* stream);
+
+/* ---- AOL rescaling (muon.py:776-785; no counterpart kernel in the reference, which leaves
+ *      these tensor expressions to torch.compile) ------------------------------------------- */
+/* Rows each block of the two launches below covers (one wavefront per row). */
+int muon_amd_aol_rows_per_block(void);
+/* Host-side check of the tables: row_prefix_host[nmat+1] counts blocks over the rows of each
+ * Gram matrix, seg_prefix_host[3*nmat+1] over the rows of X, X^T and A of each matrix.        */
+int muon_amd_validate_aol(const MuonAolDesc* descs_host, int nmat, const int32_t* row_prefix_host,
+                          const int32_t* seg_prefix_host);
+/* rvec_i = max(bf16(sum_j |A_ij|), eps)^-1/2 for every row of every Gram matrix.             */
+int muon_amd_aol_rowsum(const MuonAolDesc* descs_dev, const int32_t* row_prefix_dev, int nmat,
+                        int nblocks, float eps, void* stream);
+/* X <- diag(r) X in both stored orientations and A <- diag(r) A diag(r), in place.  The
+ * reference divides the rows of A by s = r^-2 instead (muon.py:785), which is not symmetric
+ * and, stored through its mirroring kernel, depends on the tile the autotuner picked; the
+ * symmetric form is the Gram matrix of the rescaled X that the iteration assumes.            */
+int muon_amd_aol_rescale(const MuonAolDesc* descs_dev, const int32_t* seg_prefix_dev, int nmat,
+                         int nblocks, void* stream);
 
 /* ---- auxiliary Adam (muon.py:104-109 and 255-258) ---------------------------------------- */
 /* m <- lerp(m, g, w1); v <- lerp(v, g*g, w2)  with w1 = 1-beta1, w2 = 1-beta2;

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libmuon_amd.so")
 ABI_VERSION = 1
 ROUND_REFERENCE = 1
 ROUND_FUSED = 0
+NORM_UNIT = 2
 SRC_F32 = 0
 SRC_BF16 = 1
 
@@ -38,6 +39,11 @@ ADAM_DESC = np.dtype(
      ("update", "<u8"), ("numel", "<i8"), ("dtype", "<i4"), ("reserved", "<i4")],
     align=True)
 
+AOL_DESC = np.dtype(
+    [("xr", "<u8"), ("xc", "<u8"), ("gram", "<u8"), ("rvec", "<u8"),
+     ("m_p", "<i4"), ("n_p", "<i4"), ("ld_n", "<i4"), ("ld_m", "<i4")],
+    align=True)
+
 _c_int = ctypes.c_int
 _c_float = ctypes.c_float
 _vp = ctypes.c_void_p
@@ -50,6 +56,11 @@ SIGNATURES = {
     "muon_amd_sizeof_gemm_desc": (ctypes.c_size_t, []),
     "muon_amd_sizeof_tile_job": (ctypes.c_size_t, []),
     "muon_amd_sizeof_adam_desc": (ctypes.c_size_t, []),
+    "muon_amd_sizeof_aol_desc": (ctypes.c_size_t, []),
+    "muon_amd_aol_rows_per_block": (_c_int, []),
+    "muon_amd_validate_aol": (_c_int, [_vp, _c_int, _vp, _vp]),
+    "muon_amd_aol_rowsum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _vp]),
+    "muon_amd_aol_rescale": (_c_int, [_vp, _vp, _c_int, _c_int, _vp]),
     "muon_amd_elementwise_block_elems": (_c_int, []),
     "muon_amd_normalize_tile": (_c_int, []),
     "muon_amd_gemm_tile_rows": (_c_int, [_c_int]),
@@ -90,7 +101,8 @@ def load():
     if lib.muon_amd_abi_version() != ABI_VERSION:
         raise MuonAmdError(f"ABI mismatch: library {lib.muon_amd_abi_version()}, binding {ABI_VERSION}")
     for dt, fn in ((MAT_DESC, lib.muon_amd_sizeof_mat_desc), (GEMM_DESC, lib.muon_amd_sizeof_gemm_desc),
-                   (TILE_JOB, lib.muon_amd_sizeof_tile_job), (ADAM_DESC, lib.muon_amd_sizeof_adam_desc)):
+                   (TILE_JOB, lib.muon_amd_sizeof_tile_job), (ADAM_DESC, lib.muon_amd_sizeof_adam_desc),
+                   (AOL_DESC, lib.muon_amd_sizeof_aol_desc)):
         if dt.itemsize != fn():
             raise MuonAmdError(f"struct layout mismatch: binding {dt.itemsize} bytes, library {fn()}")
     _lib = lib

@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmuon_amd.so")
-SOURCES = ["capi.hip", "elementwise.hip", "ns_gemm.hip"]
+SOURCES = ["capi.hip", "elementwise.hip", "aol.hip", "ns_gemm.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # hipcc -O3 must not form packed-fp32 instructions on this target

@@ -214,7 +214,9 @@ __global__ __launch_bounds__(64) void norm_finalize_kernel(const MuonMatDesc* __
     if (threadIdx.x == 0) {
         float nrm = sqrtf(s);
         float den;
-        if (round_reference) {
+        if (round_reference == 2) {
+            den = 1.f;                     // no pre-scale: the AOL variant rescales by rows instead
+        } else if (round_reference) {
             nrm = round_bf(nrm);           // the norm of a bf16 tensor is a bf16 tensor
             den = round_bf(nrm + eps);     // bf16 tensor + python scalar -> bf16 tensor
         } else {
@@ -539,7 +541,7 @@ int muon_amd_norm_finalize(const MuonMatDesc* descs_dev, int nmat, float eps, in
     MUON_REQUIRE(nmat > 0, "norm_finalize: nmat=%d", nmat);
     hipLaunchKernelGGL(norm_finalize_kernel, dim3(nmat), dim3(64), 0,
                        static_cast<hipStream_t>(stream), descs_dev, eps,
-                       (flags & MUON_AMD_ROUND_REFERENCE) ? 1 : 0);
+                       (flags & MUON_AMD_NORM_UNIT) ? 2 : ((flags & MUON_AMD_ROUND_REFERENCE) ? 1 : 0));
     return check_launch("norm_finalize");
 }
 

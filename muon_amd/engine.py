@@ -62,6 +62,13 @@ class _ChunkRuntime:
         parts = [gemm.reshape(-1).view(np.uint8), chunk.sym_jobs.view(np.uint8),
                  chunk.full_jobs.view(np.uint8), chunk.block_prefix.view(np.uint8),
                  chunk.tile_prefix.view(np.uint8)]
+        if chunk.variant == "aol4":
+            aol = chunk.aol_descs(base)
+            _lib.check(lib.muon_amd_validate_aol(_lib.host_ptr(aol), chunk.nmat,
+                                                 _lib.host_ptr(chunk.aol_row_prefix),
+                                                 _lib.host_ptr(chunk.aol_seg_prefix)), "validate_aol")
+            parts += [aol.view(np.uint8), chunk.aol_row_prefix.view(np.uint8),
+                      chunk.aol_seg_prefix.view(np.uint8)]
         offs, blob, cur = [], [], 0
         for p in parts:
             offs.append(cur)
@@ -77,6 +84,8 @@ class _ChunkRuntime:
         self.full_jobs_ptr = b + offs[2]
         self.block_prefix_ptr = b + offs[3]
         self.tile_prefix_ptr = b + offs[4]
+        if chunk.variant == "aol4":
+            self.aol_ptr, self.aol_row_prefix_ptr, self.aol_seg_prefix_ptr = (b + o for o in offs[5:8])
         self.mat_dev = None
         self.mat_key = None
 
@@ -117,8 +126,9 @@ class _ChunkRuntime:
         _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
             int(mutate_grad), s), "momentum"))
+        norm_flags = flags | (_lib.NORM_UNIT if c.variant == "aol4" else 0)
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
-            mats, c.nmat, eps, flags, s), "norm_finalize"))
+            mats, c.nmat, eps, norm_flags, s), "norm_finalize"))
         _launch("normalize", elts * 2 + padded * 4, lambda: _lib.check(lib.muon_amd_normalize(
             mats, self.tile_prefix_ptr, c.nmat, c.ntiles, s), "normalize"))
         flops = {
@@ -126,17 +136,27 @@ class _ChunkRuntime:
             _plan.PH_POLY: sum(lay.m * lay.m * (lay.m + 1) for lay in c.layouts),
         }
         f_upd = sum(2 * lay.m * lay.m * lay.n for lay in c.layouts)
+
+        def gemm(name, ph, it, jobs_ptr, njobs, work):
+            al, be, ga = c.phase_scalars(ph, it)
+            _launch(name, work, lambda: _lib.check(lib.muon_amd_ns_gemm(
+                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags, s), "ns_gemm"))
+
         for it in range(c.steps):
-            for ph, name in ((_plan.PH_SYRK, "ns_gemm/syrk"), (_plan.PH_POLY, "ns_gemm/poly")):
-                al, be, ga = c.phase_scalars(ph)
-                _launch(name, flops[ph], lambda ph=ph, al=al, be=be, ga=ga: _lib.check(lib.muon_amd_ns_gemm(
-                    self.gemm_ptr[ph], self.sym_jobs_ptr, len(c.sym_jobs), c.tile_class, al, be, ga,
-                    flags, s), "ns_gemm"))
+            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_SYRK])
+            if c.variant == "aol4" and it == 0:
+                # muon.py:776-785: row sums of |A|, then X and A rescaled in place (A becomes the
+                # Gram matrix of the rescaled X, so this iteration needs no second X X^T)
+                gram_bytes = sum(lay.mp * lay.mp * 2 for lay in c.layouts)
+                _launch("aol_rowsum", gram_bytes, lambda: _lib.check(lib.muon_amd_aol_rowsum(
+                    self.aol_ptr, self.aol_row_prefix_ptr, c.nmat, int(c.aol_row_prefix[-1]), eps, s),
+                    "aol_rowsum"))
+                _launch("aol_rescale", 2 * gram_bytes + 8 * padded, lambda: _lib.check(lib.muon_amd_aol_rescale(
+                    self.aol_ptr, self.aol_seg_prefix_ptr, c.nmat, int(c.aol_seg_prefix[-1]), s),
+                    "aol_rescale"))
+            gemm("ns_gemm/poly", _plan.PH_POLY, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_POLY])
             ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
-            al, be, ga = c.phase_scalars(ph)
-            _launch("ns_gemm/update", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm(
-                self.gemm_ptr[ph], self.full_jobs_ptr, len(c.full_jobs), c.tile_class, al, be, ga,
-                flags, s), "ns_gemm"))
+            gemm("ns_gemm/update", ph, it, self.full_jobs_ptr, len(c.full_jobs), f_upd)
         _launch("apply", apply_bytes, lambda: _lib.check(lib.muon_amd_apply(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply"))
 
@@ -148,12 +168,12 @@ class MuonGroupEngine:
     """
 
     def __init__(self, shapes, device, steps: int = 5, reference_rounding: bool = True,
-                 workspace_cap: int | None = None):
+                 workspace_cap: int | None = None, variant: str = "ns5"):
         _lib.load()
         self.device = torch.device(device)
         self.shapes = [(int(r), int(c)) for r, c in shapes]
         cap = DEFAULT_WORKSPACE_CAP if workspace_cap is None else int(workspace_cap)
-        self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap)
+        self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap, variant)
         ws_bytes = max(c.workspace_bytes for c in self.chunks)
         self.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self.device)
         base = self.workspace.data_ptr()

@@ -8,6 +8,7 @@ import torch
 
 from . import _lib
 from .engine import AdamGroupEngine, MuonGroupEngine, require_gpu_tensor
+from .plan import AOL_COEFFS
 
 _ROUNDINGS = {"reference": True, "fused": False}
 _ENGINE_CACHE: "OrderedDict[tuple, object]" = OrderedDict()
@@ -45,17 +46,9 @@ def _src_dtype(t: torch.Tensor) -> int:
     raise TypeError(f"unsupported dtype {t.dtype}")
 
 
-def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float = 1e-7, *,
-                                rounding: str = "reference") -> torch.Tensor:
-    """Newton-Schulz orthogonalisation of G (reference muon.py:265-291): bf16 result of the
-    shape of G; leading dimensions are a batch.
-
-    rounding="reference" rounds to bf16 wherever the reference's bf16 tensor expression does;
-    "fused" rounds once per stored matrix (closer to the fp32 result).
-    """
+def _orthogonalise(G: torch.Tensor, steps: int, epsilon: float, ref: bool, variant: str) -> torch.Tensor:
     assert G.ndim >= 2                                     # muon.py:275
     require_gpu_tensor(G, "G")
-    ref = _rounding_flag(rounding)
     if G.dtype not in (torch.float32, torch.bfloat16):
         G = G.float()
     G = G.contiguous()
@@ -65,8 +58,8 @@ def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float 
     if G.numel() == 0:
         return out
     with torch.cuda.device(G.device):
-        eng = _cached(("ns", G.device, rows, cols, batch, int(steps), ref),
-                      lambda: MuonGroupEngine([(rows, cols)] * batch, G.device, int(steps), ref))
+        eng = _cached(("ns", G.device, rows, cols, batch, int(steps), ref, variant),
+                      lambda: MuonGroupEngine([(rows, cols)] * batch, G.device, int(steps), ref, variant=variant))
         gsz, osz = rows * cols * G.element_size(), rows * cols * 2
         eng.run([G.data_ptr() + b * gsz for b in range(batch)], [0] * batch, [0] * batch,
                 [out.data_ptr() + b * osz for b in range(batch)], [1.0] * batch,
@@ -75,8 +68,34 @@ def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float 
     return out
 
 
+def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float = 1e-7, *,
+                                rounding: str = "reference") -> torch.Tensor:
+    """Newton-Schulz orthogonalisation of G (reference muon.py:265-291): bf16 result of the
+    shape of G; leading dimensions are a batch.
+
+    rounding="reference" rounds to bf16 wherever the reference's bf16 tensor expression does;
+    "fused" rounds once per stored matrix (closer to the fp32 result).
+    """
+    return _orthogonalise(G, steps, epsilon, _rounding_flag(rounding), "ns5")
+
+
+def zeropower_via_aol4(G: torch.Tensor, epsilon: float = 1e-7) -> torch.Tensor:
+    """The 4-iteration variant with AOL rescaling (reference muon.py:748-799): instead of the
+    Frobenius pre-scale, the rows of X are divided by sqrt(sum_j |(X X^T)_ij|), which bounds the
+    spectral norm by 1 and starts closer to orthogonal; four quintic iterations with the
+    coefficients of muon.py:754-759 follow, the first reusing the rescaled Gram matrix.
+
+    One deliberate difference: the Gram matrix is rescaled on both sides (it then is the Gram
+    matrix of the rescaled X); the reference divides its rows only (muon.py:785), which is not
+    symmetric, depends on its autotuned tile through its mirroring store, and loses the
+    contraction of the iteration for matrices with uneven row norms.
+    """
+    return _orthogonalise(G, len(AOL_COEFFS), epsilon, False, "aol4")
+
+
 def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
-                nesterov: bool = True, ns_steps: int = 5, *, rounding: str = "reference") -> torch.Tensor:
+                nesterov: bool = True, ns_steps: int = 5, *, rounding: str = "reference",
+                ns_variant: str = "ns5") -> torch.Tensor:
     """Reference muon.py:8-15.  Updates `momentum` in place, overwrites `grad` with the Nesterov
     blend (as the reference's grad.lerp_ does) and returns the scaled bf16 orthogonalised update
     (2-D for 4-D conv filters, else the shape of grad)."""
@@ -100,8 +119,9 @@ def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
     if grad.numel() == 0:
         return out
     with torch.cuda.device(grad.device):
-        eng = _cached(("ns", grad.device, rows, cols, batch, int(ns_steps), ref),
-                      lambda: MuonGroupEngine([(rows, cols)] * batch, grad.device, int(ns_steps), ref))
+        eng = _cached(("ns", grad.device, rows, cols, batch, int(ns_steps), ref, ns_variant),
+                      lambda: MuonGroupEngine([(rows, cols)] * batch, grad.device, int(ns_steps), ref,
+                                              variant=ns_variant))
         gsz, osz = rows * cols * grad.element_size(), rows * cols * 2
         eng.run([grad.data_ptr() + b * gsz for b in range(batch)],
                 [momentum.data_ptr() + b * gsz for b in range(batch)], [0] * batch,

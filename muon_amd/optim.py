@@ -24,7 +24,10 @@ def _world_size() -> int:
 class _MuonBase(torch.optim.Optimizer):
     """Shared machinery: engine caches and the two per-group update paths."""
 
-    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes):
+    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5"):
+        if ns_variant not in ("ns5", "aol4"):
+            raise ValueError(f"ns_variant must be 'ns5' or 'aol4', got {ns_variant!r}")
+        self._ns_variant = ns_variant
         self._reference_rounding = _rounding_flag(ns_rounding)
         self._mutate_grad = bool(mutate_grad)
         self._workspace_bytes = workspace_bytes
@@ -107,7 +110,8 @@ class _MuonBase(torch.optim.Optimizer):
         eng = self._muon_engines.get(key)
         if eng is None:
             self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
-            eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes)
+            eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes,
+                                  variant=self._ns_variant)
             self._muon_engines[key] = eng
         n = len(shapes)
         with torch.cuda.device(device):
@@ -163,14 +167,16 @@ class SingleDeviceMuon(_MuonBase):
 
     Keyword-only extras (not in the reference): ns_rounding ("reference" | "fused"),
     mutate_grad (write the Nesterov blend back into p.grad as the reference's in-place lerp does;
-    off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace).
+    off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace),
+    ns_variant ("ns5": the five-iteration specification muon.py:265-291; "aol4": the
+    four-iteration AOL-rescaled variant muon.py:748-799, see zeropower_via_aol4).
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
-                 mutate_grad=False, workspace_bytes=None):
+                 mutate_grad=False, workspace_bytes=None, ns_variant="ns5"):
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
         super().__init__(params, defaults)
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -220,10 +226,11 @@ class SingleDeviceMuonWithAuxAdam(_MuonBase):
 
     _SORT_MUON = False
 
-    def __init__(self, param_groups, *, ns_rounding="reference", mutate_grad=False, workspace_bytes=None):
+    def __init__(self, param_groups, *, ns_rounding="reference", mutate_grad=False, workspace_bytes=None,
+                 ns_variant="ns5"):
         _fill_aux_adam_groups(param_groups, self._SORT_MUON)
         super().__init__(param_groups, dict())
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant)
 
     @torch.no_grad()
     def step(self, closure=None):

@@ -21,6 +21,11 @@ import numpy as np
 from . import _lib
 
 NS_COEFFS = (3.4445, -4.7750, 2.0315)   # reference muon.py:276
+# per-iteration coefficients of the 4-iteration AOL-rescaled variant, reference muon.py:754-759
+AOL_COEFFS = ((4.0098, -7.0585, 2.4635), (3.4585, -5.5479, 2.5959),
+              (2.7573, -3.2939, 1.4254), (2.7215, -3.0494, 1.3169))
+VARIANTS = ("ns5", "aol4")
+AOL_ROWS = 4                            # must match muon_amd_aol_rows_per_block()
 TILE_DIMS = {0: (128, 128), 1: (256, 256)}   # must match muon_amd_gemm_tile_rows/cols()
 # output tiles (rows, cols) of one XCD-resident super-block: as many tiles as an XCD holds workgroups
 SUPER_DIMS = {0: (8, 8), 1: (4, 8)}
@@ -132,8 +137,12 @@ def xcd_permutation(njobs: int, group: int = 32) -> np.ndarray:
 class ChunkPlan:
     """Layout, descriptor tables and tile job lists of one chunk."""
 
-    def __init__(self, mats, tile_class: int, steps: int, reference_rounding: bool):
+    def __init__(self, mats, tile_class: int, steps: int, reference_rounding: bool, variant: str = "ns5"):
         # mats: list of (index, rows, cols)
+        assert variant in VARIANTS
+        if variant == "aol4":           # fixed schedule, one rounding per stored matrix
+            steps, reference_rounding = len(AOL_COEFFS), False
+        self.variant = variant
         self.tile_class = tile_class
         self.tile_rows, self.tile_cols = TILE_DIMS[tile_class]
         self.tile = pad_unit(tile_class)          # padding unit of the chunk
@@ -165,6 +174,15 @@ class ChunkPlan:
         off += _round_up(self.nblocks * 4, _ALIGN)
         self.off_denoms = off
         off += _round_up(self.nmat * 4, _ALIGN)
+        # AOL variant: r = s^-1/2 per row of each Gram matrix, and the block prefixes of its two launches
+        self.off_rvec = []
+        for lay in self.layouts:
+            self.off_rvec.append(off)
+            off += _round_up(lay.mp * 4, _ALIGN) if variant == "aol4" else 0
+        rowblk = [lay.mp // AOL_ROWS for lay in self.layouts]
+        self.aol_row_prefix = np.concatenate([[0], np.cumsum(rowblk)]).astype(np.int32)
+        segblk = [b for lay in self.layouts for b in (lay.mp // AOL_ROWS, lay.np_ // AOL_ROWS, lay.mp // AOL_ROWS)]
+        self.aol_seg_prefix = np.concatenate([[0], np.cumsum(segblk)]).astype(np.int32)
         self.workspace_bytes = off
         self.sym_jobs = self._jobs(sym=True)
         self.full_jobs = self._jobs(sym=False)
@@ -266,9 +284,21 @@ class ChunkPlan:
             r["scale"] = 1.0
         return d
 
-    def phase_scalars(self, phase: int):
-        """(alpha, beta, gamma) of the GEMM epilogue for a phase."""
-        a, b, c = NS_COEFFS
+    def aol_descs(self, base: int) -> np.ndarray:
+        """MuonAolDesc table: after the normalise launch X is in `X` and X^T in `XT0`."""
+        d = np.zeros(self.nmat, dtype=_lib.AOL_DESC)
+        for k, lay in enumerate(self.layouts):
+            r = d[k]
+            r["xr"] = base + lay.off["X"]
+            r["xc"] = base + lay.off["XT0"]
+            r["gram"] = base + lay.off["A"]
+            r["rvec"] = base + self.off_rvec[k]
+            r["m_p"], r["n_p"], r["ld_n"], r["ld_m"] = lay.mp, lay.np_, lay.ldn, lay.ldm
+        return d
+
+    def phase_scalars(self, phase: int, iteration: int = 0):
+        """(alpha, beta, gamma) of the GEMM epilogue for a phase of an iteration."""
+        a, b, c = AOL_COEFFS[iteration] if self.variant == "aol4" else NS_COEFFS
         if phase == PH_SYRK:
             return 1.0, 0.0, c
         if phase == PH_POLY:
@@ -276,7 +306,7 @@ class ChunkPlan:
         return 1.0, a, 0.0
 
 
-def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int):
+def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5"):
     """Split matrices [(rows, cols), ...] into chunks of one tile class each whose workspace stays
     under `workspace_cap` bytes (a single matrix larger than the cap gets a chunk of its own).
     Same-shape matrices are kept together so that their tiles batch into full waves of the GPU."""
@@ -289,13 +319,13 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
         tc = tile_class_for(min(rows, cols))
         need = matrix_workspace_bytes(rows, cols, pad_unit(tc))
         if cur and (tc != cur_class or cur_bytes + need > workspace_cap):
-            chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding))
+            chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding, variant))
             cur, cur_bytes = [], 0
         cur.append((i, rows, cols))
         cur_bytes += need
         cur_class = tc
     if cur:
-        chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding))
+        chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding, variant))
     return chunks
 
 

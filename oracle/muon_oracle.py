@@ -10,6 +10,9 @@ implementation (all citations are into /root/reference/muon.py):
                              3.4445, -4.7750, 2.0315, transpose-if-tall, bf16 storage)
   ns5_fp64_closed_form       the same map written through the SVD in float64:
                              U diag(p^steps(sigma / ||G||_F)) V^T, p(x) = a x + b x^3 + c x^5
+  ns_aol4                    muon.py:748-799  (the live 4-iteration variant with AOL rescaling,
+                             built on the Triton kernels muon.py:349-746; see its docstring
+                             for what of it can and cannot be pinned)
   muon_update                muon.py:8-15
   adam_update                muon.py:104-109
   OracleSingleDeviceMuon     muon.py:73-101
@@ -27,7 +30,22 @@ What pins each function (the reference ships no tests, golden vectors or fixture
                      recurrences for several steps, the conv-shape aspect-ratio rule.
   * adam_update   -- equals torch.optim.AdamW step for step; first-step closed form g/(|g|+eps).
   * step classes  -- behavioural unit tests written from the cited lines.
-No function here is "parity unpinned".
+  * ns_aol4       -- PARITY UNPINNED against the reference's live code: that variant only
+                     runs through Triton kernels under torch.compile on a GPU (neither can
+                     run where this oracle is written), its rounding points are chosen by the
+                     compiler's fusion, and its `A / s` (muon.py:785) divides the rows of the
+                     Gram matrix only, which is not symmetric: stored through the mirroring
+                     kernel (muon.py:538-552) the result depends on the autotuned tile and
+                     triangle, and in float64 the iteration then diverges for matrices with
+                     uneven row norms (tests/test_oracle.py shows it).  ns_aol4 restates the
+                     variant with the Gram matrix rescaled on both sides, diag(r) A diag(r) --
+                     the Gram matrix of the rescaled X, which is what the derivation of the
+                     iteration assumes.  That map is pinned by an independent closed form
+                     (ns_aol4_closed_form: the SVD of diag(r) X with the chain of the four
+                     quintics applied to its singular values), by orthogonal and diagonal
+                     inputs (both reduce to the scalar chain at 1), the AOL bound
+                     sigma_max(diag(r) X) <= 1, the transpose rule and batched == per-matrix.
+No other function here is "parity unpinned".
 """
 from __future__ import annotations
 
@@ -55,6 +73,67 @@ def _ns5(G: torch.Tensor, steps: int, eps: float, work_dtype: torch.dtype) -> to
     if tall:                                              # muon.py:289-290
         X = X.mT
     return X
+
+
+# muon.py:754-759
+AOL_CONSTS = ((4.0098, -7.0585, 2.4635), (3.4585, -5.5479, 2.5959),
+              (2.7573, -3.2939, 1.4254), (2.7215, -3.0494, 1.3169))
+
+
+def _upper_mirrored(F: torch.Tensor) -> torch.Tensor:
+    """What a kernel that computes the blocks on or above the diagonal and stores each block and
+    its transpose leaves in memory (muon.py:414-423, 538-552), taken to the limit of 1 x 1 blocks."""
+    return torch.triu(F) + torch.triu(F, 1).mT
+
+
+def ns_aol4(G: torch.Tensor, epsilon: float = 1e-7, work_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """The 4-iteration AOL-rescaled variant, muon.py:748-799, with the Gram matrix rescaled on
+    both sides (see the module docstring).  Every Triton kernel of the reference accumulates in
+    fp32 and rounds once at its store (muon.py:411-412, 531-536, 701-702); the pointwise torch
+    expressions between them are taken in fp32 with one rounding at each stored tensor, as the
+    compiler the reference runs them through fuses them.  With work_dtype=float64 nothing rounds."""
+    assert G.ndim >= 2
+    acc = torch.float64 if work_dtype == torch.float64 else torch.float32
+    X = G.to(work_dtype)                                           # muon.py:760
+    tall = G.size(-2) > G.size(-1)
+    if tall:                                                       # muon.py:761-762
+        X = X.mT
+    gram = lambda Y: _upper_mirrored((Y.to(acc) @ Y.to(acc).mT).to(work_dtype))      # ns_line_1
+    A = gram(X)                                                    # muon.py:778
+    s = torch.clamp_min(A.to(acc).abs().sum(dim=-1, keepdim=True).to(work_dtype).to(acc), epsilon)  # muon.py:779-781
+    r = torch.rsqrt(s)
+    X = (X.to(acc) * r).to(work_dtype)                             # muon.py:782
+    A = (A.to(acc) * (r * r.mT)).to(work_dtype)                    # muon.py:785, on both sides
+    for it, (a, b, c) in enumerate(AOL_CONSTS):
+        if it > 0:
+            A = gram(X)                                            # muon.py:792
+        Af = A.to(acc)
+        B = _upper_mirrored((c * (Af @ Af.mT) + b * Af).to(work_dtype))               # ns_line_2, muon.py:786, 793
+        X = (a * X.to(acc) + B.to(acc) @ X.to(acc)).to(work_dtype)                    # ns_line_3, muon.py:787, 794
+    if tall:                                                       # muon.py:797-798
+        X = X.mT
+    return X
+
+
+def ns_aol4_closed_form(G, epsilon: float = 1e-7) -> np.ndarray:
+    """The same map through the SVD, in float64: with Y = diag(r) X = U diag(sigma) V^T every
+    iteration acts on the singular values only, so the result is U diag(q3(q2(q1(q0(sigma))))) V^T."""
+    G = np.asarray(G, dtype=np.float64)
+    tall = G.shape[-2] > G.shape[-1]
+    X = np.swapaxes(G, -1, -2) if tall else G
+    A = X @ np.swapaxes(X, -1, -2)
+    s = np.maximum(np.abs(A).sum(axis=-1, keepdims=True), epsilon)
+    U, sig, Vt = np.linalg.svd(X / np.sqrt(s), full_matrices=False)
+    out = (U * aol_poly_chain(sig)[..., None, :]) @ Vt
+    return np.swapaxes(out, -1, -2) if tall else out
+
+
+def aol_poly_chain(x):
+    """q3(q2(q1(q0(x)))) for the four quintics of muon.py:754-759, elementwise in float64."""
+    x = np.asarray(x, dtype=np.float64)
+    for a, b, c in AOL_CONSTS:
+        x = a * x + b * x ** 3 + c * x ** 5
+    return x
 
 
 def ns5_bf16(G: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.Tensor:
@@ -91,13 +170,15 @@ def ns5_fp64_closed_form(G, steps: int = 5, eps: float = 1e-7) -> np.ndarray:
 # Update rules
 # --------------------------------------------------------------------------------------
 def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
-                nesterov: bool = True, ns_steps: int = 5) -> torch.Tensor:
-    """muon.py:8-15.  Mutates `momentum` and (with nesterov) `grad` exactly as the reference."""
+                nesterov: bool = True, ns_steps: int = 5, ns=None) -> torch.Tensor:
+    """muon.py:8-15.  Mutates `momentum` and (with nesterov) `grad` exactly as the reference.
+    `ns` replaces the orthogonalisation (muon.py:13 calls whichever zeropower_via_newtonschulz5
+    the module defines: the specification by default here, ns_aol4 for the live variant)."""
     momentum.lerp_(grad, 1 - beta)                                        # muon.py:9
     update = grad.lerp_(momentum, beta) if nesterov else momentum         # muon.py:10
     if update.ndim == 4:                                                  # muon.py:11-12
         update = update.view(len(update), -1)
-    update = ns5_bf16(update, ns_steps)                                   # muon.py:13
+    update = ns5_bf16(update, ns_steps) if ns is None else ns(update)     # muon.py:13
     update *= max(1, grad.size(-2) / grad.size(-1)) ** 0.5                # muon.py:14
     return update
 
@@ -117,9 +198,10 @@ def adam_update(grad, buf1, buf2, step, betas, eps):
 class OracleSingleDeviceMuon(torch.optim.Optimizer):
     """muon.py:73-101."""
 
-    def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95):
+    def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, ns=None):
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
         super().__init__(params, defaults)
+        self.ns = ns
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -139,7 +221,8 @@ def _muon_param_step(opt, p, group):
     state = opt.state[p]
     if len(state) == 0:                                                    # muon.py:95-96
         state["momentum_buffer"] = torch.zeros_like(p)
-    update = muon_update(p.grad, state["momentum_buffer"], beta=group["momentum"])  # :97
+    update = muon_update(p.grad, state["momentum_buffer"], beta=group["momentum"],
+                         ns=getattr(opt, "ns", None))                      # muon.py:97
     p.mul_(1 - group["lr"] * group["weight_decay"])                        # muon.py:98
     p.add_(update.reshape(p.shape), alpha=-group["lr"])                    # muon.py:99
 
@@ -162,7 +245,8 @@ def _adam_param_step(opt, p, group):
 class OracleSingleDeviceMuonWithAuxAdam(torch.optim.Optimizer):
     """muon.py:202-260."""
 
-    def __init__(self, param_groups):
+    def __init__(self, param_groups, ns=None):
+        self.ns = ns
         for group in param_groups:
             assert "use_muon" in group
             if group["use_muon"]:

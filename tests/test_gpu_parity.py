@@ -516,3 +516,47 @@ def test_bf16_functional_updates(M):
     _assert_bf16_close(got, want, 5e-3, "adam direction")
     _assert_bf16_close(b1g, b1c, 2e-3, "exp_avg")
     _assert_bf16_close(b2g, b2c, 2e-3, "exp_avg_sq")
+
+
+# ------------------------------------------------------------------------------------------
+# The 4-iteration AOL-rescaled variant (muon.py:748-799).  Parity with the reference's live code
+# is unpinned (see the oracle's header); the oracle restatement is pinned by its SVD closed form.
+# ------------------------------------------------------------------------------------------
+AOL_SHAPES = [((768, 3072), 1e-3), ((3072, 768), 1e-3), ((768, 768), 1e-3), ((1024, 4096), 1e-4),
+              ((64, 216), 1e-2), ((512, 2304), 1e-2), ((128, 16384), 1e-2), ((130, 300), 1.0), ((5, 3), 1.0)]
+
+
+@pytest.mark.parametrize("shape,std", AOL_SHAPES)
+def test_aol4_matches_oracle_and_closed_form(M, shape, std):
+    torch.manual_seed(hash(shape) % 1000)
+    G = torch.randn(*shape) * std * (torch.rand(shape[0], 1) * 3 + 0.05)       # uneven row norms
+    got = M.zeropower_via_aol4(_dev(G))
+    assert got.dtype == torch.bfloat16 and got.shape == G.shape
+    got = got.float().cpu()
+    assert O.rel_fro(got, O.ns_aol4(G).float()) <= TOL_BF16
+    assert O.rel_fro(got.double(), O.ns_aol4_closed_form(G.bfloat16().double().numpy())) <= TOL_FP32
+
+
+def test_aol4_batched_special_inputs_and_optimizer_step(M):
+    torch.manual_seed(1320)
+    Gb = torch.randn(5, 96, 160) * 1e-2
+    got = M.zeropower_via_aol4(_dev(Gb))
+    per = torch.stack([M.zeropower_via_aol4(_dev(g)) for g in Gb])
+    assert torch.equal(got, per)                                       # batched == per matrix, bit for bit
+    assert torch.count_nonzero(M.zeropower_via_aol4(torch.zeros(40, 24, device="cuda"))) == 0
+    Q, _ = torch.linalg.qr(torch.randn(64, 64, dtype=torch.float64))
+    out = M.zeropower_via_aol4(_dev(Q.float())).double().cpu()
+    assert O.rel_fro(out, float(O.aol_poly_chain(1.0)) * Q) <= TOL_BF16   # orthogonal input -> chain(1) * Q
+    # optimizer classes with ns_variant="aol4" against the oracle classes using ns_aol4
+    shapes = [(256, 384), (384, 256), (16, 8, 3, 3), (2, 64, 96)]
+    cpu, gpu = _clone_params(shapes, 0.02, 1321)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns=O.ns_aol4)
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns_variant="aol4")
+    for step in range(2):
+        _set_grads(cpu, gpu, 1e-2)
+        oc.step()
+        og.step()
+        for pc, pg in zip(cpu, gpu):
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 2e-3, (tuple(pc.shape), step)
+    with pytest.raises(ValueError):
+        M.SingleDeviceMuon(gpu, ns_variant="aol5")

@@ -217,3 +217,27 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, os.path.join(dirpath, f)
     assert "oracle" not in open(os.path.join(ROOT, "muon.py")).read()
+
+
+def test_aol_variant_plan_validates():
+    """The 4-iteration variant: fixed schedule, one rounding per stored matrix, row-scale vectors
+    in the workspace, and block prefixes the library accepts."""
+    lib = _lib.load()
+    assert lib.muon_amd_aol_rows_per_block() == plan.AOL_ROWS
+    assert _lib.AOL_DESC.itemsize == lib.muon_amd_sizeof_aol_desc() == 48
+    chunks = plan.plan_chunks(SHAPES, 5, True, 1 << 30, "aol4")
+    for c in chunks:
+        assert c.variant == "aol4" and c.steps == len(plan.AOL_COEFFS) == 4 and not c.reference_rounding
+        d = c.aol_descs(1 << 20)
+        rc = lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix),
+                                       _lib.host_ptr(c.aol_seg_prefix))
+        assert rc == 0, lib.muon_amd_last_error()
+        assert [c.phase_scalars(plan.PH_POLY, it) for it in range(4)] == [(co[2], co[1], 0.0) for co in plan.AOL_COEFFS]
+        assert c.phase_scalars(plan.PH_UPD_EVEN, 2) == (1.0, plan.AOL_COEFFS[2][0], 0.0)
+        for k, l in enumerate(c.layouts):      # the r vectors lie inside the workspace, apart from everything else
+            assert c.off_denoms + 4 * c.nmat <= c.off_rvec[k] and c.off_rvec[k] + 4 * l.mp <= c.workspace_bytes
+        bad = c.aol_seg_prefix.copy()
+        bad[1] += 1
+        assert lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix), _lib.host_ptr(bad)) == -1
+    ns5 = plan.plan_chunks(SHAPES, 5, True, 1 << 30)
+    assert all(a.workspace_bytes > b.workspace_bytes for a, b in zip(chunks, ns5))

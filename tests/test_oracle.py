@@ -243,3 +243,79 @@ def test_oracle_reproduces_golden_fixtures(golden_dir):
         np.testing.assert_allclose(O.ns5_fp32(G).numpy(), z[n + "/fp32"], rtol=1e-6, atol=1e-7)
         if G.ndim == 2:
             assert O.rel_fro(z[n + "/fp32"], z[n + "/fp64_closed_form"]) < 2e-4
+
+
+# ------------------------------------------------------------------------------------------
+# The 4-iteration AOL-rescaled variant (muon.py:748-799)
+# ------------------------------------------------------------------------------------------
+def _uneven_rows(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    G = torch.randn(*shape, dtype=torch.float64, generator=g)
+    return G * (torch.rand(*shape[:-1], 1, dtype=torch.float64, generator=g) * 3 + 0.05)
+
+
+@pytest.mark.parametrize("shape", [(64, 96), (96, 64), (128, 128), (30, 200), (3, 40, 24)])
+def test_aol4_matches_its_svd_closed_form(shape):
+    G = _uneven_rows(shape, 77)
+    want = O.ns_aol4_closed_form(G.numpy())
+    assert O.rel_fro(O.ns_aol4(G, work_dtype=torch.float64), want) < 1e-12
+    assert O.rel_fro(O.ns_aol4(G.float(), work_dtype=torch.float32).double(), want) < 1e-5
+    assert O.rel_fro(O.ns_aol4(G.float()).double(), want) < 2e-2          # bf16 storage
+    # transpose rule (muon.py:761-762, 797-798; a square matrix is never transposed, and the row
+    # rescaling is not symmetric in rows and columns) and batching
+    if shape[-2] != shape[-1]:
+        assert O.rel_fro(O.ns_aol4(G.mT.contiguous(), work_dtype=torch.float64).mT, want) < 1e-12
+    if G.ndim == 3:
+        per = torch.stack([O.ns_aol4(g, work_dtype=torch.float64) for g in G])
+        assert O.rel_fro(per, want) < 1e-12
+
+
+def test_aol4_special_inputs_reduce_to_the_scalar_chain():
+    chain1 = float(O.aol_poly_chain(1.0))
+    assert abs(chain1 - (-0.9935212261846591)) < 1e-12      # the first quintic is negative above 0.884
+    Q, _ = torch.linalg.qr(torch.randn(48, 48, dtype=torch.float64, generator=torch.Generator().manual_seed(5)))
+    # orthogonal input: A = I, s = 1, every singular value is 1
+    assert (O.ns_aol4(Q, work_dtype=torch.float64) - chain1 * Q).abs().max() < 1e-12
+    # diagonal input: A = diag(d^2), s = d^2, the rescaled matrix is diag(sign d)
+    d = torch.tensor([0.5, -2.0, 3.0, 0.1], dtype=torch.float64)
+    got = O.ns_aol4(torch.diag(d), work_dtype=torch.float64)
+    assert (got - torch.diag(chain1 * torch.sign(d))).abs().max() < 1e-12
+    assert torch.count_nonzero(O.ns_aol4(torch.zeros(8, 12))) == 0
+
+
+def test_aol_rescaling_bounds_the_spectral_norm_and_the_band():
+    for seed, shape in enumerate([(64, 96), (200, 30), (128, 128)]):
+        G = _uneven_rows(shape, 100 + seed)
+        X = G.mT if shape[0] > shape[1] else G
+        s = (X @ X.mT).abs().sum(-1, keepdim=True)
+        assert torch.linalg.svdvals(X * torch.rsqrt(s)).max() <= 1 + 1e-12      # AOL bound
+        sv = torch.linalg.svdvals(O.ns_aol4(G, work_dtype=torch.float64))
+        assert sv.max() < 1.25                                                   # stays in the attracting band
+    # the scalar chain maps [0.03, 0.86] into a tight band around 1 (the first quintic has a root
+    # at 0.884: larger singular values change sign)
+    y = O.aol_poly_chain(np.linspace(0.03, 0.86, 400))
+    assert y.min() > 0.98 and y.max() < 1.02
+    assert O.aol_poly_chain(0.92) < -0.9
+
+
+def test_row_only_rescaling_of_the_gram_matrix_is_not_a_contraction():
+    """Why ns_aol4 rescales the Gram matrix on both sides: `A / s` (muon.py:785) divides rows
+    only; with the mirrored store of the polynomial kernel (muon.py:538-552, either triangle,
+    muon.py:493-495) the iteration leaves the attracting band for matrices with uneven row norms."""
+    def rows_only(G, upper):
+        X = G.clone()
+        A = X @ X.mT
+        s = A.abs().sum(-1, keepdim=True).clamp_min(1e-7)
+        X = X * torch.rsqrt(s)
+        A = A / s
+        for it, (a, b, c) in enumerate(O.AOL_CONSTS):
+            if it > 0:
+                A = X @ X.mT
+            F = c * (A @ A.mT) + b * A
+            B = torch.triu(F) + torch.triu(F, 1).mT if upper else torch.tril(F) + torch.tril(F, -1).mT
+            X = a * X + B @ X
+        return torch.linalg.svdvals(X).max().item()
+
+    G = _uneven_rows((30, 200), 3)
+    assert rows_only(G, True) > 10 and rows_only(G, False) > 10
+    assert torch.linalg.svdvals(O.ns_aol4(G, work_dtype=torch.float64)).max() < 1.25
