@@ -70,7 +70,7 @@ def mat2d(shape):
 # ------------------------------------------------------------------------------------------
 # GPU leg
 # ------------------------------------------------------------------------------------------
-def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5"):
+def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False):
     import muon_amd
     from muon_amd import engine
 
@@ -91,7 +91,7 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5"):
     opt = muon_amd.SingleDeviceMuonWithAuxAdam([
         dict(params=pm, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01),
         dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)],
-        ns_variant=ns_variant)
+        ns_variant=ns_variant, use_graph=use_graph)
 
     # The gradients stay resident and unchanged over the run (the step does not write them); the
     # momentum and the parameters move every step, so every step orthogonalises new matrices.
@@ -103,13 +103,13 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5"):
 
     # timed region: exactly `steps` steps back to back, one synchronisation on either side; a pair
     # of HIP events on the launch stream brackets every kernel launch inside it
-    engine.PROFILE = []
+    engine.PROFILE = None if use_graph else []      # a replayed graph has no per-launch events
     t0 = time.perf_counter()
     for _ in range(steps):
         opt.step()
     torch.cuda.synchronize()
     total_ms = (time.perf_counter() - t0) * 1e3
-    prof, engine.PROFILE = engine.PROFILE, None
+    prof, engine.PROFILE = engine.PROFILE or [], None
 
     per_label = {}
     for label, work, e0, e1 in prof:
@@ -200,6 +200,9 @@ def main():
                     help="ns5: the five-iteration specification (the headline); aol4: the 4-iteration "
                          "AOL-rescaled variant (its flop count is 11/15 of the headline's, so only the step "
                          "time of such a run is comparable, not the roofline fraction)")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the Muon launches from a HIP graph (use_graph=True): step time only, the "
+                         "per-kernel figures need the eager launches")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary GPT-2 measurement")
     ap.add_argument("--copy-probe", action="store_true",
@@ -221,7 +224,14 @@ def main():
         b.copy_(a)                                                            # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del a, b
-    res = run_optimizer_workload(args.workload, steps, warmup, seed=1234 + 4, ns_variant=args.ns_variant)
+    res = run_optimizer_workload(args.workload, steps, warmup, seed=1234 + 4, ns_variant=args.ns_variant,
+                                 use_graph=args.graph)
+    if args.graph:
+        print(json.dumps({"metric": f"muon_step_ms_{args.workload}", "value": round(res["ms_per_step"], 3),
+                          "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                          "ms_per_step": round(res["ms_per_step"], 3), "higher_is_better": False,
+                          "config": {"workload": args.workload, "ns_variant": args.ns_variant, "launch": "hip graph replay"}}))
+        return
     kernels, gemm_work, gemm_ms, gemm_n = summarize_kernels(res["per_label"])
     ew_bytes = sum(w for l, (w, ms, n) in res["per_label"].items() if not l.startswith("ns_gemm"))
     ew_ms = sum(ms for l, (w, ms, n) in res["per_label"].items() if not l.startswith("ns_gemm"))
@@ -271,7 +281,9 @@ def main():
     if not args.no_extra and args.workload == "llama3-8b":
         g = run_optimizer_workload("gpt2-124m", 10, 3, seed=1234 + 2)
         _, gw, gms, _ = summarize_kernels(g["per_label"])
-        line["gpt2_124m"] = {"ms_per_step": round(g["ms_per_step"], 3), "ns_tflops_sym": round(gw / gms / 1e9, 1)}
+        gg = run_optimizer_workload("gpt2-124m", 10, 3, seed=1234 + 2, use_graph=True)
+        line["gpt2_124m"] = {"ms_per_step": round(g["ms_per_step"], 3), "ns_tflops_sym": round(gw / gms / 1e9, 1),
+                             "ms_per_step_graph_replay": round(gg["ms_per_step"], 3)}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.workload)
         if line["cpu_baseline"]["value"]:

@@ -132,6 +132,10 @@ typedef struct MuonAolDesc {
 
 int         muon_amd_abi_version(void);
 const char* muon_amd_last_error(void);
+/* One-time set-up on the current device (raises the dynamic LDS limit of the GEMM kernels).
+ * Optional -- the first GEMM launch does it too -- but required before recording launches
+ * into a HIP graph, because it is not a stream operation.                                   */
+int         muon_amd_init(void);
 
 /* sizeof() of the structs above, so that a binding can check its own layout. */
 size_t muon_amd_sizeof_mat_desc(void);
@@ -167,10 +171,14 @@ int muon_amd_validate_mats(const MuonMatDesc* descs_host, int nmat,
  *   momentum <- lerp(momentum, grad, one_minus_beta);
  *   u = nesterov ? lerp(grad, momentum, beta) : momentum       (lerp = torch's two-branch rule)
  * With mutate_grad != 0 and nesterov, u is also written back into grad as the reference does.
- * A matrix whose descriptor has momentum == NULL is only cast (u = grad).                    */
+ * A matrix whose descriptor has momentum == NULL is only cast (u = grad).
+ * scalars_dev (here and in muon_amd_apply / muon_amd_adam): NULL, or device memory holding the
+ * float arguments of the call in their order ({one_minus_beta, beta} here), which the kernel then
+ * reads at run time in place of the by-value ones -- a launch recorded into a HIP graph can so
+ * be replayed with new hyper-parameters after a small copy into that memory.               */
 int muon_amd_momentum(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
                       int nblocks, float one_minus_beta, float beta, int nesterov,
-                      int mutate_grad, void* stream);
+                      int mutate_grad, const float* scalars_dev, void* stream);
 
 /* denom = ||u||_F + eps per matrix from the partial sums (muon.py:282).  Under
  * MUON_AMD_ROUND_REFERENCE the norm and the sum are rounded to bf16 as the reference's bf16
@@ -191,7 +199,8 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
 /* result -> update = bf16(result * scale) (muon.py:14);  if param: param <- param*wd_factor
  * - lr*update (muon.py:98-99); if out: out <- update (what muon_update returns, muon.py:15). */
 int muon_amd_apply(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
-                   int nblocks, float lr, float wd_factor, void* stream);
+                   int nblocks, float lr, float wd_factor, const float* scalars_dev /* {lr, wd_factor} */,
+                   void* stream);
 
 /* ---- AOL rescaling (muon.py:776-785; no counterpart kernel in the reference, which leaves
  *      these tensor expressions to torch.compile) ------------------------------------------- */
@@ -218,7 +227,9 @@ int muon_amd_aol_rescale(const MuonAolDesc* descs_dev, const int32_t* seg_prefix
  * (as the reference's Python does) and passed rounded to float. */
 int muon_amd_adam(const MuonAdamDesc* descs_dev, const int32_t* block_prefix_dev, int ntensors,
                   int nblocks, float lr, float wd_factor, float w1, float w2, float eps,
-                  float bias1, float bias2, void* stream);
+                  float bias1, float bias2,
+                  const float* scalars_dev /* {lr, wd_factor, w1, w2, eps, bias1, bias2} */,
+                  void* stream);
 
 #ifdef __cplusplus
 }

@@ -52,6 +52,7 @@ _vp = ctypes.c_void_p
 SIGNATURES = {
     "muon_amd_abi_version": (_c_int, []),
     "muon_amd_last_error": (ctypes.c_char_p, []),
+    "muon_amd_init": (_c_int, []),
     "muon_amd_sizeof_mat_desc": (ctypes.c_size_t, []),
     "muon_amd_sizeof_gemm_desc": (ctypes.c_size_t, []),
     "muon_amd_sizeof_tile_job": (ctypes.c_size_t, []),
@@ -67,13 +68,13 @@ SIGNATURES = {
     "muon_amd_gemm_tile_cols": (_c_int, [_c_int]),
     "muon_amd_validate_gemm": (_c_int, [_vp, _c_int, _vp, _c_int, _c_int]),
     "muon_amd_validate_mats": (_c_int, [_vp, _c_int, _vp, _vp, _c_int]),
-    "muon_amd_momentum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _vp]),
+    "muon_amd_momentum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _vp, _vp]),
     "muon_amd_norm_finalize": (_c_int, [_vp, _c_int, _c_float, _c_int, _vp]),
     "muon_amd_normalize": (_c_int, [_vp, _vp, _c_int, _c_int, _vp]),
     "muon_amd_ns_gemm": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _vp]),
-    "muon_amd_apply": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _vp]),
+    "muon_amd_apply": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _vp, _vp]),
     "muon_amd_adam": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_float,
-                               _c_float, _c_float, _c_float, _vp]),
+                               _c_float, _c_float, _c_float, _vp, _vp]),
 }
 
 

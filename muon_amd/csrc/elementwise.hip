@@ -187,10 +187,16 @@ __device__ __forceinline__ float momentum_block(const MuonMatDesc& d, int64_t bl
     return ss;
 }
 
+// `sc` (optional, device memory): {one_minus_beta, beta} read at run time instead of the by-value
+// arguments, so that a captured launch can be replayed with new hyper-parameters.
 __global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
     const MuonMatDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, float w,
-    float beta, int nesterov, int mutate_grad) {
+    float beta, int nesterov, int mutate_grad, const float* __restrict__ sc) {
     __shared__ float red[4];
+    if (sc) {
+        w = sc[0];
+        beta = sc[1];
+    }
     const int b = blockIdx.x;
     const int mi = find_segment(prefix, nmat, b);
     const MuonMatDesc d = descs[mi];
@@ -366,9 +372,15 @@ __device__ __forceinline__ void apply_block(const MuonMatDesc& d, int64_t block_
     }
 }
 
+// `sc` (optional, device memory): {lr, wd_factor} read at run time instead of the arguments.
 __global__ __launch_bounds__(EW_THREADS) void apply_kernel(const MuonMatDesc* __restrict__ descs,
                                                             const int32_t* __restrict__ prefix,
-                                                            int nmat, float neg_lr, float wd_factor) {
+                                                            int nmat, float neg_lr, float wd_factor,
+                                                            const float* __restrict__ sc) {
+    if (sc) {
+        neg_lr = -sc[0];
+        wd_factor = sc[1];
+    }
     const int b = blockIdx.x;
     const int mi = find_segment(prefix, nmat, b);
     const MuonMatDesc d = descs[mi];
@@ -461,7 +473,17 @@ __global__ __launch_bounds__(EW_THREADS) void adam_kernel(const MuonAdamDesc* __
                                                            const int32_t* __restrict__ prefix,
                                                            int ntensors, float neg_lr,
                                                            float wd_factor, float w1, float w2,
-                                                           float eps, float bias1, float bias2) {
+                                                           float eps, float bias1, float bias2,
+                                                           const float* __restrict__ sc) {
+    if (sc) {   // {lr, wd_factor, w1, w2, eps, bias1, bias2} read at run time instead of the arguments
+        neg_lr = -sc[0];
+        wd_factor = sc[1];
+        w1 = sc[2];
+        w2 = sc[3];
+        eps = sc[4];
+        bias1 = sc[5];
+        bias2 = sc[6];
+    }
     const int b = blockIdx.x;
     const int ti = find_segment(prefix, ntensors, b);
     const MuonAdamDesc d = descs[ti];
@@ -526,12 +548,12 @@ int muon_amd_validate_mats(const MuonMatDesc* descs, int nmat, const int32_t* bl
 
 int muon_amd_momentum(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
                       int nblocks, float one_minus_beta, float beta, int nesterov,
-                      int mutate_grad, void* stream) {
+                      int mutate_grad, const float* scalars_dev, void* stream) {
     MUON_REQUIRE(descs_dev && block_prefix_dev, "momentum: null table");
     MUON_REQUIRE(nmat > 0 && nblocks > 0, "momentum: nmat=%d nblocks=%d", nmat, nblocks);
     hipLaunchKernelGGL(momentum_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
                        static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, nmat,
-                       one_minus_beta, beta, nesterov, mutate_grad);
+                       one_minus_beta, beta, nesterov, mutate_grad, scalars_dev);
     return check_launch("momentum");
 }
 
@@ -555,24 +577,24 @@ int muon_amd_normalize(const MuonMatDesc* descs_dev, const int32_t* tile_prefix_
 }
 
 int muon_amd_apply(const MuonMatDesc* descs_dev, const int32_t* block_prefix_dev, int nmat,
-                   int nblocks, float lr, float wd_factor, void* stream) {
+                   int nblocks, float lr, float wd_factor, const float* scalars_dev, void* stream) {
     MUON_REQUIRE(descs_dev && block_prefix_dev, "apply: null table");
     MUON_REQUIRE(nmat > 0 && nblocks > 0, "apply: nmat=%d nblocks=%d", nmat, nblocks);
     hipLaunchKernelGGL(apply_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
                        static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, nmat, -lr,
-                       wd_factor);
+                       wd_factor, scalars_dev);
     return check_launch("apply");
 }
 
 int muon_amd_adam(const MuonAdamDesc* descs_dev, const int32_t* block_prefix_dev, int ntensors,
                   int nblocks, float lr, float wd_factor, float w1, float w2, float eps,
-                  float bias1, float bias2, void* stream) {
+                  float bias1, float bias2, const float* scalars_dev, void* stream) {
     MUON_REQUIRE(descs_dev && block_prefix_dev, "adam: null table");
     MUON_REQUIRE(ntensors > 0 && nblocks > 0, "adam: ntensors=%d nblocks=%d", ntensors, nblocks);
-    MUON_REQUIRE(bias1 != 0.f && bias2 != 0.f, "adam: zero bias correction");
+    MUON_REQUIRE(scalars_dev || (bias1 != 0.f && bias2 != 0.f), "adam: zero bias correction");
     hipLaunchKernelGGL(adam_kernel, dim3(nblocks), dim3(EW_THREADS), 0,
                        static_cast<hipStream_t>(stream), descs_dev, block_prefix_dev, ntensors,
-                       -lr, wd_factor, w1, w2, eps, bias1, bias2);
+                       -lr, wd_factor, w1, w2, eps, bias1, bias2, scalars_dev);
     return check_launch("adam");
 }
 

@@ -450,12 +450,14 @@ static const TileClass kTileClasses[kNumTileClasses] = {
     {Cfg1::BM, Cfg1::BN, Cfg1::NT, Cfg1::LDS_BYTES},
 };
 
+// The kernels use more dynamic LDS than the default limit: raised once per process and device
+// function (not a stream operation, so it must not wait for the first launch, which may be one
+// that a caller records into a HIP graph).
 template <typename Cfg>
-static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
-                       float beta, float gamma, int flags, hipStream_t s) {
+static int raise_lds_limit() {
     static bool attr_set = false;
-    auto kern = ns_gemm_kernel<Cfg>;
     if (!attr_set) {
+        auto kern = ns_gemm_kernel<Cfg>;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
                                 static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
@@ -464,8 +466,16 @@ static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int n
         }
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs, alpha, beta,
-                       gamma, flags);
+    return MUON_AMD_OK;
+}
+
+template <typename Cfg>
+static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
+                       float beta, float gamma, int flags, hipStream_t s) {
+    const int rc = raise_lds_limit<Cfg>();
+    if (rc != MUON_AMD_OK) return rc;
+    hipLaunchKernelGGL(ns_gemm_kernel<Cfg>, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                       alpha, beta, gamma, flags);
     return check_launch("ns_gemm");
 }
 
@@ -474,6 +484,11 @@ static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int n
 using namespace muon_amd;
 
 extern "C" {
+
+int muon_amd_init(void) {
+    const int rc = raise_lds_limit<Cfg0>();
+    return rc != MUON_AMD_OK ? rc : raise_lds_limit<Cfg1>();
+}
 
 int muon_amd_gemm_tile_rows(int tile_class) {
     MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "gemm_tile_rows: unknown tile class %d", tile_class);

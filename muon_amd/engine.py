@@ -40,10 +40,15 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def _upload(arr: np.ndarray, device) -> torch.Tensor:
-    """Async host->device copy of a table through pinned staging (no stream or host sync)."""
-    host = torch.from_numpy(arr.view(np.uint8).reshape(-1)).pin_memory()
-    return host.to(device, non_blocking=True)
+def _upload(arr: np.ndarray, device, into: torch.Tensor | None = None) -> torch.Tensor:
+    """Async host->device copy of a table through pinned staging (no stream or host sync).
+    With `into`, the bytes land in that existing device buffer, whose address launches recorded
+    in a HIP graph keep referring to."""
+    host = torch.from_numpy(np.ascontiguousarray(arr).view(np.uint8).reshape(-1)).pin_memory()
+    if into is None:
+        return host.to(device, non_blocking=True)
+    into.copy_(host, non_blocking=True)
+    return into
 
 
 class _ChunkRuntime:
@@ -106,14 +111,18 @@ class _ChunkRuntime:
                                               _lib.host_ptr(self.chunk.block_prefix),
                                               _lib.host_ptr(self.chunk.tile_prefix), self.chunk.tile),
                    "validate_mats")
-        self.mat_dev = _upload(d, self.device)
+        self.mat_dev = _upload(d, self.device, into=self.mat_dev)
         self.mat_key = key
         self.src_dtypes = list(src_dtypes)
 
-    def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor):
+    def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor, scalars_ptr=0):
+        """Enqueue the chunk's launches.  scalars_ptr: device address of {one_minus_beta, beta, lr,
+        wd_factor}, read by the kernels at run time in place of the by-value arguments."""
         lib = _lib.load()
         c = self.chunk
         s = _stream_ptr(self.device)
+        sc_mom = scalars_ptr or None
+        sc_apply = scalars_ptr + 8 if scalars_ptr else None
         flags = _lib.ROUND_REFERENCE if c.reference_rounding else _lib.ROUND_FUSED
         mats = self.mat_dev.data_ptr()
         elts = sum(lay.numel for lay in c.layouts)
@@ -125,7 +134,7 @@ class _ChunkRuntime:
         apply_bytes = sum(lay.numel * (2 * sz + 2) for lay, sz in zip(c.layouts, store))
         _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
-            int(mutate_grad), s), "momentum"))
+            int(mutate_grad), sc_mom, s), "momentum"))
         norm_flags = flags | (_lib.NORM_UNIT if c.variant == "aol4" else 0)
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
             mats, c.nmat, eps, norm_flags, s), "norm_finalize"))
@@ -158,7 +167,7 @@ class _ChunkRuntime:
             ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
             gemm("ns_gemm/update", ph, it, self.full_jobs_ptr, len(c.full_jobs), f_upd)
         _launch("apply", apply_bytes, lambda: _lib.check(lib.muon_amd_apply(
-            mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, s), "apply"))
+            mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, sc_apply, s), "apply"))
 
 
 class MuonGroupEngine:
@@ -168,9 +177,14 @@ class MuonGroupEngine:
     """
 
     def __init__(self, shapes, device, steps: int = 5, reference_rounding: bool = True,
-                 workspace_cap: int | None = None, variant: str = "ns5"):
-        _lib.load()
+                 workspace_cap: int | None = None, variant: str = "ns5", use_graph: bool = False):
         self.device = torch.device(device)
+        with torch.cuda.device(self.device):
+            _lib.check(_lib.load().muon_amd_init(), "init")
+        self.use_graph = bool(use_graph)
+        self._graph = None
+        self._graph_key = None
+        self._scalars = torch.zeros(4, dtype=torch.float32, device=self.device)
         self.shapes = [(int(r), int(c)) for r, c in shapes]
         cap = DEFAULT_WORKSPACE_CAP if workspace_cap is None else int(workspace_cap)
         self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap, variant)
@@ -189,7 +203,25 @@ class MuonGroupEngine:
             idx = [lay.index for lay in rt.chunk.layouts]
             rt.bind([grads[i] for i in idx], [momenta[i] for i in idx], [params[i] for i in idx],
                     [outs[i] for i in idx], [scales[i] for i in idx], [src_dtypes[i] for i in idx])
-            rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor)
+        if not self.use_graph or PROFILE is not None:
+            for rt in self.runtimes:
+                rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor)
+            return
+        # Graph mode: every launch of the step is recorded once into a HIP graph and replayed.
+        # What changes between steps lives in device memory that the recorded launches read: the
+        # matrix descriptors (tensor addresses; rewritten in place by bind() when one moved) and
+        # the hyper-parameter scalars, refreshed here by a small copy ahead of the replay.
+        _upload(np.array([one_minus_beta, beta, lr, wd_factor], dtype=np.float32), self.device,
+                into=self._scalars.view(torch.uint8))
+        key = (bool(nesterov), bool(mutate_grad), float(eps))
+        if self._graph is None or key != self._graph_key:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for rt in self.runtimes:
+                    rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor,
+                           scalars_ptr=self._scalars.data_ptr())
+            self._graph, self._graph_key = graph, key
+        self._graph.replay()
 
 
 class AdamGroupEngine:
@@ -228,4 +260,4 @@ class AdamGroupEngine:
         nbytes = sum(n * (14 if t == _lib.SRC_BF16 else 28) for n, t in zip(self.numels, dtypes))
         _launch("adam", nbytes, lambda: _lib.check(lib.muon_amd_adam(
             self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels), self.nblocks, lr,
-            1 - lr * weight_decay, w1, w2, eps, bias1, bias2, _stream_ptr(self.device)), "adam"))
+            1 - lr * weight_decay, w1, w2, eps, bias1, bias2, None, _stream_ptr(self.device)), "adam"))

@@ -24,7 +24,8 @@ def _world_size() -> int:
 class _MuonBase(torch.optim.Optimizer):
     """Shared machinery: engine caches and the two per-group update paths."""
 
-    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5"):
+    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5", use_graph=False):
+        self._use_graph = bool(use_graph)
         if ns_variant not in ("ns5", "aol4"):
             raise ValueError(f"ns_variant must be 'ns5' or 'aol4', got {ns_variant!r}")
         self._ns_variant = ns_variant
@@ -111,7 +112,7 @@ class _MuonBase(torch.optim.Optimizer):
         if eng is None:
             self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
             eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes,
-                                  variant=self._ns_variant)
+                                  variant=self._ns_variant, use_graph=self._use_graph)
             self._muon_engines[key] = eng
         n = len(shapes)
         with torch.cuda.device(device):
@@ -169,14 +170,17 @@ class SingleDeviceMuon(_MuonBase):
     mutate_grad (write the Nesterov blend back into p.grad as the reference's in-place lerp does;
     off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace),
     ns_variant ("ns5": the five-iteration specification muon.py:265-291; "aol4": the
-    four-iteration AOL-rescaled variant muon.py:748-799, see zeropower_via_aol4).
+    four-iteration AOL-rescaled variant muon.py:748-799, see zeropower_via_aol4), use_graph
+    (record the launches of a Muon group's step into a HIP graph once and replay it every step;
+    tensor addresses and hyper-parameters are read from device memory, so gradients may be
+    reallocated and learning rates scheduled between steps).
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
-                 mutate_grad=False, workspace_bytes=None, ns_variant="ns5"):
+                 mutate_grad=False, workspace_bytes=None, ns_variant="ns5", use_graph=False):
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
         super().__init__(params, defaults)
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -227,10 +231,10 @@ class SingleDeviceMuonWithAuxAdam(_MuonBase):
     _SORT_MUON = False
 
     def __init__(self, param_groups, *, ns_rounding="reference", mutate_grad=False, workspace_bytes=None,
-                 ns_variant="ns5"):
+                 ns_variant="ns5", use_graph=False):
         _fill_aux_adam_groups(param_groups, self._SORT_MUON)
         super().__init__(param_groups, dict())
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph)
 
     @torch.no_grad()
     def step(self, closure=None):

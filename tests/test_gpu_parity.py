@@ -560,3 +560,43 @@ def test_aol4_batched_special_inputs_and_optimizer_step(M):
             assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 2e-3, (tuple(pc.shape), step)
     with pytest.raises(ValueError):
         M.SingleDeviceMuon(gpu, ns_variant="aol5")
+
+
+# ------------------------------------------------------------------------------------------
+# HIP-graph replay of a Muon group's step
+# ------------------------------------------------------------------------------------------
+def test_graph_replay_equals_eager_every_step(M):
+    """use_graph=True records the launches once and replays them; every replay is compared bit for
+    bit with the eager optimizer, with eager work and synchronisations between the replays,
+    gradients that are reallocated each step, a learning rate that changes each step, and a
+    second pair of optimizers whose matrices fill more than one chunk."""
+    for shapes, cap in (([(768, 768), (256, 384), (384, 256), (16, 8, 3, 3)], None),
+                        ([(512, 640), (640, 512), (300, 200)], 3 << 20)):
+        torch.manual_seed(1330)
+        base = [torch.randn(*s) * 0.02 for s in shapes]
+        pe = [torch.nn.Parameter(_dev(b.clone())) for b in base]
+        pg = [torch.nn.Parameter(_dev(b.clone())) for b in base]
+        ae, ag = torch.nn.Parameter(torch.ones(33, device="cuda")), torch.nn.Parameter(torch.ones(33, device="cuda"))
+        mk = lambda pm, pa, g: M.SingleDeviceMuonWithAuxAdam(
+            [dict(params=pm, use_muon=True, lr=0.02, weight_decay=0.01), dict(params=[pa], use_muon=False, weight_decay=0.01)],
+            use_graph=g, workspace_bytes=cap)
+        oe, og = mk(pe, ae, False), mk(pg, ag, True)
+        for step in range(5):
+            lr = 0.02 * (1 - 0.15 * step)
+            oe.param_groups[0]["lr"] = og.param_groups[0]["lr"] = lr
+            for a, b in zip(pe + [ae], pg + [ag]):
+                g = torch.randn_like(a) * 1e-2
+                a.grad, b.grad = g.clone(), g.clone()        # new gradient tensors every step
+            oe.step()
+            og.step()
+            junk = torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")    # eager work between replays
+            torch.cuda.synchronize()
+            for a, b in zip(pe + [ae], pg + [ag]):
+                assert torch.equal(a.detach(), b.detach()), (shapes, step)
+            for a, b in zip(pe, pg):
+                assert torch.equal(oe.state[a]["momentum_buffer"], og.state[b]["momentum_buffer"]), (shapes, step)
+            oe.zero_grad(set_to_none=True)
+            og.zero_grad(set_to_none=True)
+            del junk
+        eng = next(iter(og._muon_engines.values()))
+        assert eng._graph is not None and (cap is None or len(eng.runtimes) > 1)

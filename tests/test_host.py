@@ -45,10 +45,10 @@ def test_struct_layouts_match_the_library():
 def test_entry_points_reject_bad_arguments_without_a_gpu():
     lib = _lib.load()
     assert lib.muon_amd_ns_gemm(None, None, 1, 0, 1.0, 0.0, 0.0, 0, None) == -1
-    assert lib.muon_amd_momentum(None, None, 1, 1, 0.05, 0.95, 1, 0, None) == -1
-    assert lib.muon_amd_adam(None, None, 1, 1, 1e-3, 1.0, 0.1, 0.05, 1e-10, 0.1, 0.05, None) == -1
+    assert lib.muon_amd_momentum(None, None, 1, 1, 0.05, 0.95, 1, 0, None, None) == -1
+    assert lib.muon_amd_adam(None, None, 1, 1, 1e-3, 1.0, 0.1, 0.05, 1e-10, 0.1, 0.05, None, None) == -1
     with pytest.raises(_lib.MuonAmdError):
-        _lib.check(lib.muon_amd_apply(None, None, 0, 0, 0.0, 1.0, None), "apply")
+        _lib.check(lib.muon_amd_apply(None, None, 0, 0, 0.0, 1.0, None, None), "apply")
 
 
 # ------------------------------------------------------------------------------------------
