@@ -100,12 +100,19 @@ typedef struct MuonGemmDesc {
     int32_t rows, colsn;                /* padded extent of the output (multiples of the tile) */
 } MuonGemmDesc;
 
-/* One output tile of one matrix. */
+/* One output tile of one matrix, or one share of its reduction.  A tile whose K is long and
+ * whose launch would leave most of the GPU idle (the one 128 x 128 tile of X X^T for a
+ * 128 x 16384 matrix) is given to `count` jobs, each reducing k0..k1; each parks its fp32
+ * accumulators in slot part_base + index of the split workspace, and the job that arrives last
+ * adds the slots in slot order and writes the tile (the result does not depend on arrival order). */
 typedef struct MuonTileJob {
-    int32_t desc;   /* index into the MuonGemmDesc table of the launch */
-    int32_t i0;     /* first output row  (multiple of the tile rows)   */
-    int32_t j0;     /* first output col  (multiple of the tile cols)   */
-    int32_t diag;   /* 1 when a mirrored (symmetric) GEMM's tile lies in a diagonal block */
+    int32_t desc;      /* index into the MuonGemmDesc table of the launch */
+    int32_t i0;        /* first output row  (multiple of the tile rows)   */
+    int32_t j0;        /* first output col  (multiple of the tile cols)   */
+    int32_t diag;      /* 1 when a mirrored (symmetric) GEMM's tile lies in a diagonal block */
+    int32_t k0, k1;    /* reduction range of this job, multiples of 64; 0 and K when unsplit */
+    int32_t part_base; /* first slot of the tile's split group (also its counter); unused when unsplit */
+    int32_t split;     /* 0 when unsplit, else index | (count << 16) */
 } MuonTileJob;
 
 /* One tensor of the auxiliary Adam group. */
@@ -159,7 +166,8 @@ int muon_amd_gemm_tile_cols(int tile_class);
 /* ---- host-side validation (no GPU work): checks host copies of the tables a launch will
  *      use against what the kernels assume.  Call before uploading them.                 ---- */
 int muon_amd_validate_gemm(const MuonGemmDesc* descs_host, int ndesc,
-                           const MuonTileJob* jobs_host, int njobs, int tile_class);
+                           const MuonTileJob* jobs_host, int njobs, int tile_class,
+                           int split_slots /* slots of the split workspace the jobs may use */);
 int muon_amd_validate_mats(const MuonMatDesc* descs_host, int nmat,
                            const int32_t* block_prefix_host, const int32_t* tile_prefix_host,
                            int tile_edge);
@@ -191,10 +199,12 @@ int muon_amd_norm_finalize(const MuonMatDesc* descs_dev, int nmat, float eps, in
 int muon_amd_normalize(const MuonMatDesc* descs_dev, const int32_t* tile_prefix_dev, int nmat,
                        int ntiles, void* stream);
 
-/* One grouped GEMM launch over a tile job list (see MuonGemmDesc). */
+/* One grouped GEMM launch over a tile job list (see MuonGemmDesc).  split_partials_dev (slots of
+ * tile_rows * tile_cols floats) and split_counters_dev (one int32 per slot, zero before the
+ * first launch; every launch leaves them zero) are needed only when a job is split, else NULL. */
 int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
                      int tile_class, float alpha, float beta, float gamma, int flags,
-                     void* stream);
+                     float* split_partials_dev, int32_t* split_counters_dev, void* stream);
 
 /* result -> update = bf16(result * scale) (muon.py:14);  if param: param <- param*wd_factor
  * - lr*update (muon.py:98-99); if out: out <- update (what muon_update returns, muon.py:15). */

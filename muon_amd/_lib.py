@@ -33,7 +33,8 @@ GEMM_DESC = np.dtype(
      ("C2T", "<u8"), ("ldp", "<i4"), ("ldq", "<i4"), ("ldd", "<i4"), ("ldc", "<i4"),
      ("ldct", "<i4"), ("K", "<i4"), ("rows", "<i4"), ("colsn", "<i4")],
     align=True)
-TILE_JOB = np.dtype([("desc", "<i4"), ("i0", "<i4"), ("j0", "<i4"), ("diag", "<i4")], align=True)
+TILE_JOB = np.dtype([("desc", "<i4"), ("i0", "<i4"), ("j0", "<i4"), ("diag", "<i4"), ("k0", "<i4"),
+                     ("k1", "<i4"), ("part_base", "<i4"), ("split", "<i4")], align=True)
 ADAM_DESC = np.dtype(
     [("param", "<u8"), ("grad", "<u8"), ("exp_avg", "<u8"), ("exp_avg_sq", "<u8"),
      ("update", "<u8"), ("numel", "<i8"), ("dtype", "<i4"), ("reserved", "<i4")],
@@ -66,12 +67,12 @@ SIGNATURES = {
     "muon_amd_normalize_tile": (_c_int, []),
     "muon_amd_gemm_tile_rows": (_c_int, [_c_int]),
     "muon_amd_gemm_tile_cols": (_c_int, [_c_int]),
-    "muon_amd_validate_gemm": (_c_int, [_vp, _c_int, _vp, _c_int, _c_int]),
+    "muon_amd_validate_gemm": (_c_int, [_vp, _c_int, _vp, _c_int, _c_int, _c_int]),
     "muon_amd_validate_mats": (_c_int, [_vp, _c_int, _vp, _vp, _c_int]),
     "muon_amd_momentum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _vp, _vp]),
     "muon_amd_norm_finalize": (_c_int, [_vp, _c_int, _c_float, _c_int, _vp]),
     "muon_amd_normalize": (_c_int, [_vp, _vp, _c_int, _c_int, _vp]),
-    "muon_amd_ns_gemm": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _vp]),
+    "muon_amd_ns_gemm": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _vp, _vp]),
     "muon_amd_apply": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _vp, _vp]),
     "muon_amd_adam": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_float,
                                _c_float, _c_float, _c_float, _vp, _vp]),

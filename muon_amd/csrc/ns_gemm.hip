@@ -29,6 +29,8 @@
 
 #include "common.h"
 
+#include <vector>
+
 namespace muon_amd {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -258,8 +260,9 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 // earlier iterations) and halves 2kb+NHALF-2, 2kb+NHALF-1 (issued during this iteration into the
 // two slots block kb-1 vacated) are in flight, so the load pipe always has queued requests and
 // every request is a full 128-byte line.  NHALF = 5 fills the 160 KB LDS for the 256 x 256 tile.
-template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_>
+template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_, bool SPLIT_K_>
 struct GemmCfg {
+    static constexpr bool SPLIT_K = SPLIT_K_;     // jobs may share a tile's reduction
     static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_, NHALF = NHALF_;
     static constexpr int NW = WGM * WGN, NT = NW * 64;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
@@ -278,7 +281,8 @@ struct GemmCfg {
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, float alpha,
-    float beta, float gamma, int flags) {
+    float beta, float gamma, int flags, float* __restrict__ split_partials,
+    int32_t* __restrict__ split_counters) {
     constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
     constexpr int NHALF = Cfg::NHALF;
@@ -298,8 +302,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 #pragma unroll
     for (int j = 0; j < DPH; ++j) {
         const int r = (j * NW + wave) * 8 + (lane >> 3);
-        srcp[j] = d.P + static_cast<size_t>(i0 + r) * d.ldp + gchunk * 8;
-        srcq[j] = d.Q + static_cast<size_t>(j0 + r) * d.ldq + gchunk * 8;
+        srcp[j] = d.P + static_cast<size_t>(i0 + r) * d.ldp + job.k0 + gchunk * 8;
+        srcq[j] = d.Q + static_cast<size_t>(j0 + r) * d.ldq + job.k0 + gchunk * 8;
     }
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) uint16_t*)lds));
@@ -329,7 +333,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
 
-    const int nk = d.K / BK;
+    const int nk = (job.k1 - job.k0) / BK;      // this job's share of the reduction
     // prologue: halves 0 .. NHALF-1 = P0 Q0 P1 Q1 P2 ...
 #pragma unroll
     for (int h = 0; h < NHALF; ++h) {
@@ -424,6 +428,68 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 #undef NS_LOAD_FRAGS
 #undef NS_ISSUE_HALF
     __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
+
+    // ---- split reduction (small tile class only): a tile whose K range is shared by `count`
+    //      jobs.  Each job parks its fp32 accumulators in its own slot; the job that arrives last
+    //      adds the slots in slot order (so the sum does not depend on which job that is) and
+    //      writes the tile.  Nobody waits for anybody: the other jobs just exit.
+    //      The slots are written with device-scope stores, which go through to memory past the
+    //      XCD-private L2 (a release fence would write the whole L2 back instead); only the one
+    //      job per tile that adds them up pays for an acquire fence before its plain loads. ------
+    if constexpr (Cfg::SPLIT_K) {
+        const int split_count = job.split >> 16;
+        if (split_count > 1) {
+            constexpr size_t TILE_ELEMS = static_cast<size_t>(Cfg::BM) * Cfg::BN;
+            float* const mine = split_partials + (static_cast<size_t>(job.part_base) + (job.split & 0xffff)) * TILE_ELEMS;
+            const size_t lane_off = static_cast<size_t>(wave) * TM * TN * 16 * 64 + lane;
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        __hip_atomic_store(&mine[lane_off + ((a * TN + b) * 16 + i) * 64], acc[a][b][i],
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_waitcnt(0);                     // my slot has reached memory ...
+            __syncthreads();
+            int* const ticket = reinterpret_cast<int*>(lds);
+            if (tid == 0)                                      // ... before I am counted
+                *ticket = __hip_atomic_fetch_add(&split_counters[job.part_base], 1, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            const bool last = *ticket == split_count - 1;
+            __syncthreads();                                   // the ticket is read before LDS is reused
+            if (!last) return;
+            if (tid == 0)                                      // ready for the next launch on the stream
+                __hip_atomic_store(&split_counters[job.part_base], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); // drop what this XCD cached of the slots
+            const float* const first = split_partials + static_cast<size_t>(job.part_base) * TILE_ELEMS;
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+            // slot by slot, all of a lane's loads of one slot in flight together
+            for (int sidx = 0; sidx < split_count; ++sidx) {
+                const float* const slot = first + sidx * TILE_ELEMS;
+#pragma unroll
+                for (int a = 0; a < TM; ++a) {
+                    float t[TN][16];
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) t[b][i] = slot[lane_off + ((a * TN + b) * 16 + i) * 64];
+                    __builtin_amdgcn_sched_barrier(0);     // all of these loads go out before the first add waits
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) acc[a][b][i] += t[b][i];
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
     char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
     const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
     if (d.D) ns_epilogue_impl<true, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
@@ -437,17 +503,18 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 #define NS_CFG0_MINB 2
 #define NS_CFG0_NHALF 5
 #endif
-typedef GemmCfg<128, 2, 2, NS_CFG0_MINB, NS_CFG0_NHALF> Cfg0;
-typedef GemmCfg<256, 2, 4, 1, 5> Cfg1;
+typedef GemmCfg<128, 2, 2, NS_CFG0_MINB, NS_CFG0_NHALF, true> Cfg0;
+typedef GemmCfg<256, 2, 4, 1, 5, false> Cfg1;
 constexpr int kNumTileClasses = 2;
 
 struct TileClass {
     int bm, bn, threads;
     size_t lds_bytes;
+    bool split_k;
 };
 static const TileClass kTileClasses[kNumTileClasses] = {
-    {Cfg0::BM, Cfg0::BN, Cfg0::NT, Cfg0::LDS_BYTES},
-    {Cfg1::BM, Cfg1::BN, Cfg1::NT, Cfg1::LDS_BYTES},
+    {Cfg0::BM, Cfg0::BN, Cfg0::NT, Cfg0::LDS_BYTES, Cfg0::SPLIT_K},
+    {Cfg1::BM, Cfg1::BN, Cfg1::NT, Cfg1::LDS_BYTES, Cfg1::SPLIT_K},
 };
 
 // The kernels use more dynamic LDS than the default limit: raised once per process and device
@@ -471,11 +538,12 @@ static int raise_lds_limit() {
 
 template <typename Cfg>
 static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
-                       float beta, float gamma, int flags, hipStream_t s) {
+                       float beta, float gamma, int flags, float* split_partials,
+                       int32_t* split_counters, hipStream_t s) {
     const int rc = raise_lds_limit<Cfg>();
     if (rc != MUON_AMD_OK) return rc;
     hipLaunchKernelGGL(ns_gemm_kernel<Cfg>, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
-                       alpha, beta, gamma, flags);
+                       alpha, beta, gamma, flags, split_partials, split_counters);
     return check_launch("ns_gemm");
 }
 
@@ -501,8 +569,11 @@ int muon_amd_gemm_tile_cols(int tile_class) {
 }
 
 int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJob* jobs,
-                           int njobs, int tile_class) {
+                           int njobs, int tile_class, int split_slots) {
     MUON_REQUIRE(descs && jobs, "validate_gemm: null table");
+    MUON_REQUIRE(split_slots >= 0, "validate_gemm: split_slots=%d", split_slots);
+    std::vector<int64_t> covered(static_cast<size_t>(split_slots), 0);   // per split group: K covered, jobs seen
+    std::vector<int> seen(static_cast<size_t>(split_slots), 0);
     MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "validate_gemm: unknown tile class %d", tile_class);
     MUON_REQUIRE(ndesc > 0 && njobs > 0, "validate_gemm: ndesc=%d njobs=%d", ndesc, njobs);
     const int TR = kTileClasses[tile_class].bm, TC = kTileClasses[tile_class].bn;
@@ -534,24 +605,47 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJ
                          t.j0 + TC <= d.colsn,
                      "job %d: tile (%d,%d) outside %dx%d", j, t.i0, t.j0, d.rows, d.colsn);
         MUON_REQUIRE(t.diag == 0 || t.diag == 1, "job %d: diag=%d", j, t.diag);
+        MUON_REQUIRE(t.k0 >= 0 && t.k0 < t.k1 && t.k1 <= d.K && t.k0 % BK == 0 && t.k1 % BK == 0,
+                     "job %d: K range %d..%d of %d", j, t.k0, t.k1, d.K);
+        const int count = t.split >> 16, idx = t.split & 0xffff;
+        if (count <= 1) {
+            MUON_REQUIRE(t.split == 0 && t.k0 == 0 && t.k1 == d.K, "job %d: an unsplit job covers all of K", j);
+        } else {
+            MUON_REQUIRE(kTileClasses[tile_class].split_k, "job %d: tile class %d does not split reductions", j, tile_class);
+            MUON_REQUIRE(idx < count && t.part_base >= 0 && t.part_base + count <= split_slots,
+                         "job %d: split %d of %d at slot %d, %d slots", j, idx, count, t.part_base, split_slots);
+            covered[t.part_base] += t.k1 - t.k0;
+            seen[t.part_base] += 1;
+            if (seen[t.part_base] == count)
+                MUON_REQUIRE(covered[t.part_base] == d.K, "job %d: its split group covers %lld of K=%d", j,
+                             static_cast<long long>(covered[t.part_base]), d.K);
+            MUON_REQUIRE(seen[t.part_base] <= count, "job %d: split group at slot %d has too many jobs", j, t.part_base);
+        }
         // mirrored GEMM: only tiles whose column block is on or above the row block, and tiles
         // inside a diagonal TR x TR block (stored directly, never mirrored) are flagged
         const int cblk = t.j0 / TR * TR;
         MUON_REQUIRE(!(d.CT == d.C && d.C) || (cblk >= t.i0 && t.diag == (cblk == t.i0)),
                      "job %d: mirrored GEMM needs its column block >= row block and diag set on the diagonal block", j);
     }
+    for (int g = 0; g < split_slots; ++g)
+        MUON_REQUIRE(seen[g] == 0 || covered[g] > 0, "split group %d is inconsistent", g);
     return MUON_AMD_OK;
 }
 
 int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
                      int tile_class, float alpha, float beta, float gamma, int flags,
-                     void* stream) {
+                     float* split_partials_dev, int32_t* split_counters_dev, void* stream) {
     MUON_REQUIRE(descs_dev && jobs_dev, "ns_gemm: null table");
+    MUON_REQUIRE((split_partials_dev == nullptr) == (split_counters_dev == nullptr),
+                 "ns_gemm: split partials and counters go together");
     MUON_REQUIRE(njobs > 0, "ns_gemm: njobs=%d", njobs);
     MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "ns_gemm: unknown tile class %d", tile_class);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (tile_class == 0) return launch_gemm<Cfg0>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, s);
-    return launch_gemm<Cfg1>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, s);
+    if (tile_class == 0)
+        return launch_gemm<Cfg0>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, split_partials_dev,
+                                 split_counters_dev, s);
+    return launch_gemm<Cfg1>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, split_partials_dev,
+                             split_counters_dev, s);
 }
 
 

@@ -58,15 +58,17 @@ class _ChunkRuntime:
         self.device = device
         gemm = chunk.gemm_descs(base)
         for ph in range(5):
-            jobs = chunk.sym_jobs if ph in (_plan.PH_SYRK, _plan.PH_POLY) else chunk.full_jobs
+            jobs = (chunk.syrk_jobs if ph == _plan.PH_SYRK else
+                    chunk.sym_jobs if ph == _plan.PH_POLY else chunk.full_jobs)
             _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(gemm[ph]), chunk.nmat,
-                                                  _lib.host_ptr(jobs), len(jobs), chunk.tile_class),
+                                                  _lib.host_ptr(jobs), len(jobs), chunk.tile_class,
+                                                  chunk.split_slots if ph == _plan.PH_SYRK else 0),
                        "validate_gemm")
         self.mat_template = chunk.mat_descs(base)
         # one static device blob: gemm descs | sym jobs | full jobs | block prefix | tile prefix
         parts = [gemm.reshape(-1).view(np.uint8), chunk.sym_jobs.view(np.uint8),
                  chunk.full_jobs.view(np.uint8), chunk.block_prefix.view(np.uint8),
-                 chunk.tile_prefix.view(np.uint8)]
+                 chunk.tile_prefix.view(np.uint8), chunk.syrk_jobs.view(np.uint8)]
         if chunk.variant == "aol4":
             aol = chunk.aol_descs(base)
             _lib.check(lib.muon_amd_validate_aol(_lib.host_ptr(aol), chunk.nmat,
@@ -89,8 +91,13 @@ class _ChunkRuntime:
         self.full_jobs_ptr = b + offs[2]
         self.block_prefix_ptr = b + offs[3]
         self.tile_prefix_ptr = b + offs[4]
+        self.syrk_jobs_ptr = b + offs[5]
+        # counters of the split groups: zero now, and every launch that uses them leaves them zero
+        self.split_counters = torch.zeros(max(chunk.split_slots, 1), dtype=torch.int32, device=device)
+        self.split_partials_ptr = base + chunk.off_split_partials if chunk.split_slots else None
+        self.split_counters_ptr = self.split_counters.data_ptr() if chunk.split_slots else None
         if chunk.variant == "aol4":
-            self.aol_ptr, self.aol_row_prefix_ptr, self.aol_seg_prefix_ptr = (b + o for o in offs[5:8])
+            self.aol_ptr, self.aol_row_prefix_ptr, self.aol_seg_prefix_ptr = (b + o for o in offs[6:9])
         self.mat_dev = None
         self.mat_key = None
 
@@ -148,11 +155,14 @@ class _ChunkRuntime:
 
         def gemm(name, ph, it, jobs_ptr, njobs, work):
             al, be, ga = c.phase_scalars(ph, it)
+            split = ph == _plan.PH_SYRK
             _launch(name, work, lambda: _lib.check(lib.muon_amd_ns_gemm(
-                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags, s), "ns_gemm"))
+                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags,
+                self.split_partials_ptr if split else None, self.split_counters_ptr if split else None, s),
+                "ns_gemm"))
 
         for it in range(c.steps):
-            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_SYRK])
+            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.syrk_jobs_ptr, len(c.syrk_jobs), flops[_plan.PH_SYRK])
             if c.variant == "aol4" and it == 0:
                 # muon.py:776-785: row sums of |A|, then X and A rescaled in place (A becomes the
                 # Gram matrix of the rescaled X, so this iteration needs no second X X^T)

@@ -50,6 +50,24 @@ def tile_class_for(m: int) -> int:
     return 1 if m >= BIG_TILE_MIN_M else 0
 
 
+GEMM_BK = 64                            # k-block of the GEMM kernel: K and every job's K range are multiples
+SPLIT_MAX_M = 512                       # X X^T of a matrix this short ...
+SPLIT_MIN_KBLOCKS = 32                  # ... and at least this long (in k-blocks) is split ...
+SPLIT_KBLOCKS_PER_JOB = 16              # ... into jobs of about this many k-blocks, at most SPLIT_MAX
+SPLIT_MAX = 16
+
+
+def split_factor(mp: int, kdim: int) -> int:
+    """Into how many jobs each tile of X X^T is split along its reduction.  The rule looks at the
+    matrix alone, so its result is the same bits whatever else shares the launch: a short, very
+    wide matrix has a handful of tiles with thousands of k-blocks each (one tile with 256 for
+    128 x 16384), which one workgroup per tile would grind through while the rest of the GPU idles."""
+    kblocks = kdim // GEMM_BK
+    if mp > SPLIT_MAX_M or kblocks < SPLIT_MIN_KBLOCKS:
+        return 1
+    return max(1, min(SPLIT_MAX, kblocks // SPLIT_KBLOCKS_PER_JOB))
+
+
 def pad_unit(tile_class: int) -> int:
     return max(TILE_DIMS[tile_class])
 
@@ -183,12 +201,20 @@ class ChunkPlan:
         self.aol_row_prefix = np.concatenate([[0], np.cumsum(rowblk)]).astype(np.int32)
         segblk = [b for lay in self.layouts for b in (lay.mp // AOL_ROWS, lay.np_ // AOL_ROWS, lay.mp // AOL_ROWS)]
         self.aol_seg_prefix = np.concatenate([[0], np.cumsum(segblk)]).astype(np.int32)
+        # job lists: the symmetric products share their tiles but not their reduction length
+        # (X X^T reduces over n, the polynomial over m), and only the former is ever split
+        self.split_slots = 0
+        self.syrk_jobs = self._jobs(sym=True, reduce_over_n=True)
+        self.sym_jobs = self._jobs(sym=True, reduce_over_n=False)
+        self.full_jobs = self._jobs(sym=False, reduce_over_n=False)
+        # fp32 slots of the split jobs (scratch like the rest; the per-slot counters are not part
+        # of the workspace: they must stay zero between launches, and chunks share the workspace)
+        self.off_split_partials = off
+        off += _round_up(self.split_slots * self.tile_rows * self.tile_cols * 4, _ALIGN)
         self.workspace_bytes = off
-        self.sym_jobs = self._jobs(sym=True)
-        self.full_jobs = self._jobs(sym=False)
 
     # ---- tile job lists -----------------------------------------------------------------
-    def _jobs(self, sym: bool) -> np.ndarray:
+    def _jobs(self, sym: bool, reduce_over_n: bool) -> np.ndarray:
         TR, TC = self.tile_rows, self.tile_cols
         ratio = TR // TC
         si, sj = SUPER_DIMS[self.tile_class]
@@ -197,11 +223,22 @@ class ChunkPlan:
             mt = lay.mp // TR
             nt = (lay.mp if sym else lay.np_) // TC
             ti, tj = _tile_order(mt, nt, sym, ratio, si, sj)
-            j = np.zeros(len(ti), dtype=_lib.TILE_JOB)
+            kdim = lay.np_ if reduce_over_n else lay.mp
+            nsplit = split_factor(lay.mp, kdim) if reduce_over_n else 1
+            j = np.zeros(len(ti) * nsplit, dtype=_lib.TILE_JOB)
             j["desc"] = k
-            j["i0"] = ti * TR
-            j["j0"] = tj * TC
-            j["diag"] = (ti == tj // ratio).astype(np.int32) if sym else 0
+            j["i0"] = np.repeat(ti * TR, nsplit)
+            j["j0"] = np.repeat(tj * TC, nsplit)
+            j["diag"] = np.repeat((ti == tj // ratio).astype(np.int32), nsplit) if sym else 0
+            if nsplit == 1:
+                j["k1"] = kdim
+            else:      # k-blocks dealt as evenly as 64-wide blocks allow; one group of slots per tile
+                edges = (np.arange(nsplit + 1) * (kdim // GEMM_BK) // nsplit) * GEMM_BK
+                idx = np.tile(np.arange(nsplit), len(ti))
+                j["k0"], j["k1"] = edges[idx], edges[idx + 1]
+                j["part_base"] = self.split_slots + np.repeat(np.arange(len(ti)) * nsplit, nsplit)
+                j["split"] = idx | (nsplit << 16)
+                self.split_slots += len(ti) * nsplit
             parts.append(j)
         logical = np.concatenate(parts)
         group = int(os.environ.get("MUON_AMD_XCD_GROUP", si * sj))      # measurement knob

@@ -38,13 +38,13 @@ def test_struct_layouts_match_the_library():
     lib = _lib.load()
     assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 120
     assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 88
-    assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 16
+    assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 32
     assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 56
 
 
 def test_entry_points_reject_bad_arguments_without_a_gpu():
     lib = _lib.load()
-    assert lib.muon_amd_ns_gemm(None, None, 1, 0, 1.0, 0.0, 0.0, 0, None) == -1
+    assert lib.muon_amd_ns_gemm(None, None, 1, 0, 1.0, 0.0, 0.0, 0, None, None, None) == -1
     assert lib.muon_amd_momentum(None, None, 1, 1, 0.05, 0.95, 1, 0, None, None) == -1
     assert lib.muon_amd_adam(None, None, 1, 1, 1e-3, 1.0, 0.1, 0.05, 1e-10, 0.1, 0.05, None, None) == -1
     with pytest.raises(_lib.MuonAmdError):
@@ -68,8 +68,9 @@ def test_plans_validate_and_cover_every_tile_once(ref):
         assert all(plan.tile_class_for(l.m) == c.tile_class for l in c.layouts)
         g = c.gemm_descs(1 << 20)
         for ph in range(5):
-            jobs = c.sym_jobs if ph < 2 else c.full_jobs
-            rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class)
+            jobs = c.syrk_jobs if ph == plan.PH_SYRK else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
+            rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class,
+                                            c.split_slots if ph == plan.PH_SYRK else 0)
             assert rc == 0, lib.muon_amd_last_error()
         TR, TC = c.tile_rows, c.tile_cols
         for k, l in enumerate(c.layouts):
@@ -115,13 +116,51 @@ def test_validation_catches_a_bad_table():
     g = c.gemm_descs(1 << 20)
     bad = c.full_jobs.copy()
     bad["j0"][0] = c.layouts[0].np_          # one tile past the last column
-    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[2]), 1, _lib.host_ptr(bad), len(bad), c.tile_class) == -1
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[2]), 1, _lib.host_ptr(bad), len(bad), c.tile_class, 0) == -1
     gd = g[0].copy()
     gd["K"] = 100                            # not a multiple of the k-block
-    assert lib.muon_amd_validate_gemm(_lib.host_ptr(gd), 1, _lib.host_ptr(c.sym_jobs), len(c.sym_jobs), c.tile_class) == -1
-    low = c.sym_jobs.copy()
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(gd), 1, _lib.host_ptr(c.syrk_jobs), len(c.syrk_jobs), c.tile_class, 0) == -1
+    low = c.syrk_jobs.copy()
     low["i0"][0], low["j0"][0] = c.tile_rows, 0      # below the diagonal of a mirrored GEMM
-    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[0]), 1, _lib.host_ptr(low), len(low), c.tile_class) == -1
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[0]), 1, _lib.host_ptr(low), len(low), c.tile_class, 0) == -1
+    short = c.syrk_jobs.copy()
+    short["k1"][0] -= 64                     # an unsplit job that does not reduce over all of K
+    assert lib.muon_amd_validate_gemm(_lib.host_ptr(g[0]), 1, _lib.host_ptr(short), len(short), c.tile_class, 0) == -1
+
+
+def test_split_reduction_plan():
+    """X X^T of a short, very wide matrix is split along K by a rule that looks at the matrix alone."""
+    lib = _lib.load()
+    assert [plan.split_factor(128, 16384), plan.split_factor(512, 4608), plan.split_factor(512, 2304),
+            plan.split_factor(256, 576), plan.split_factor(768, 3072), plan.split_factor(4096, 14336)] == [16, 4, 2, 1, 1, 1]
+    c = plan.plan_chunks([(128, 16384), (16384, 128), (512, 4608), (64, 216)], 5, True, 1 << 30)[0]
+    g = c.gemm_descs(1 << 20)
+    assert c.split_slots == 16 + 16 + 10 * 4 and len(c.syrk_jobs) == c.split_slots + 1
+    assert np.all(c.sym_jobs["split"] == 0) and np.all(c.full_jobs["split"] == 0)      # only X X^T is split
+    rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[plan.PH_SYRK]), c.nmat, _lib.host_ptr(c.syrk_jobs),
+                                    len(c.syrk_jobs), c.tile_class, c.split_slots)
+    assert rc == 0, lib.muon_amd_last_error()
+    for k, l in enumerate(c.layouts):        # every tile's jobs tile [0, K) in 64-wide blocks, one slot each
+        jk = c.syrk_jobs[c.syrk_jobs["desc"] == k]
+        for i0, j0 in {(a, b) for a, b in zip(jk["i0"].tolist(), jk["j0"].tolist())}:
+            t = np.sort(jk[(jk["i0"] == i0) & (jk["j0"] == j0)], order="k0")
+            assert t["k0"][0] == 0 and t["k1"][-1] == l.np_ and np.array_equal(t["k1"][:-1], t["k0"][1:])
+            assert np.all(t["k0"] % 64 == 0) and len(t) == plan.split_factor(l.mp, l.np_)
+            if len(t) > 1:
+                assert np.array_equal(np.sort(t["split"] & 0xffff), np.arange(len(t))) and len(set(t["part_base"].tolist())) == 1
+    groups = c.syrk_jobs[c.syrk_jobs["split"] != 0]
+    slots = sorted((groups["part_base"] + (groups["split"] & 0xffff)).tolist())
+    assert slots == list(range(c.split_slots))                                        # no two jobs share a slot
+    assert c.off_split_partials + c.split_slots * c.tile_rows * c.tile_cols * 4 <= c.workspace_bytes
+    # the library refuses too few slots, a hole in a group's K range and a job counted twice
+    args = (_lib.host_ptr(g[plan.PH_SYRK]), c.nmat)
+    assert lib.muon_amd_validate_gemm(*args, _lib.host_ptr(c.syrk_jobs), len(c.syrk_jobs), c.tile_class, c.split_slots - 1) == -1
+    hole = c.syrk_jobs.copy()
+    first = np.flatnonzero(hole["split"] != 0)[0]
+    hole["k1"][first] -= 64
+    assert lib.muon_amd_validate_gemm(*args, _lib.host_ptr(hole), len(hole), c.tile_class, c.split_slots) == -1
+    twice = np.concatenate([c.syrk_jobs, c.syrk_jobs[first:first + 1]])
+    assert lib.muon_amd_validate_gemm(*args, _lib.host_ptr(twice), len(twice), c.tile_class, c.split_slots) == -1
 
 
 def test_xcd_permutation_and_result_buffer():
