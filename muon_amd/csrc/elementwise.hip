@@ -18,7 +18,7 @@ constexpr int EW_PASS_ELEMS = EW_THREADS * EW_VEC * EW_ITERS;   // 8192 elements
 #endif
 constexpr int EW_PASSES = MUON_EW_PASSES;                       // passes per block (amortise the block's set-up)
 constexpr int EW_BLOCK_ELEMS = EW_PASS_ELEMS * EW_PASSES;       // elements per block
-constexpr int NT_TILE = 64;                                     // normalise/transposing tile edge
+constexpr int NT_TILE = 128;                                    // normalise/transposing tile edge
 
 // 16-/8-byte accesses through the global address space (descriptor pointers are generic to the
 // compiler).  MUON_EW_NT adds the non-temporal hint to these streaming accesses.
@@ -235,10 +235,22 @@ __global__ __launch_bounds__(64) void norm_finalize_kernel(const MuonMatDesc* __
 // ------------------------------------------------------------------------------------------
 // normalise + transpose + zero pad:  direct = bf16(u / denom), transp = direct^T
 // ------------------------------------------------------------------------------------------
+typedef uint32_t u32x4e __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4e gld4u(const uint16_t* p) {
+    return __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4e*)(p));
+}
+__device__ __forceinline__ void gst4u(uint16_t* p, u32x4e v) {     // read again soon by the GEMMs: no hint
+    *(__attribute__((address_space(1))) u32x4e*)(p) = v;
+}
+
+// One NT_TILE x NT_TILE tile per block (256-byte row segments in both orientations).  The tile goes through LDS as 32-bit words (two columns each): a
+// thread that later reads word c of rows r .. r+7 holds 8 consecutive elements of the two
+// transposed rows 2c and 2c+1.
 __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __restrict__ descs,
                                                          const int32_t* __restrict__ prefix,
                                                          int nmat) {
-    __shared__ uint16_t tile[NT_TILE][NT_TILE + 2];
+    constexpr int PITCH = NT_TILE / 2 + 2;               // words per LDS row (even: 8-byte stores)
+    __shared__ __align__(8) uint32_t tile[NT_TILE][PITCH];
     const int b = blockIdx.x;
     const int mi = find_segment(prefix, nmat, b);
     const MuonMatDesc d = descs[mi];
@@ -249,10 +261,11 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
     const uint16_t* __restrict__ u = d.u;
     const bool vec_ok = (d.cols % 8 == 0) && aligned_to(u, 16);
 
+    constexpr int CH = NT_TILE / 8;                      // 8-element chunks per tile row
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NT_TILE * CH / 256; ++i) {
         const int q = threadIdx.x + i * 256;
-        const int r = q >> 3, cc = (q & 7) * 8;
+        const int r = q / CH, cc = (q % CH) * 8;
         const int gr = R0 + r, gc = C0 + cc;
         uint16_t v[8];
 #pragma unroll
@@ -260,12 +273,11 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
         if (gr < d.rows) {
             const int64_t off = static_cast<int64_t>(gr) * d.cols + gc;
             if (vec_ok && gc + 8 <= d.cols) {
-                const uint4 raw = *reinterpret_cast<const uint4*>(u + off);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+                const u32x4e raw = gld4u(u + off);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    v[2 * k] = static_cast<uint16_t>(w[k] & 0xffffu);
-                    v[2 * k + 1] = static_cast<uint16_t>(w[k] >> 16);
+                    v[2 * k] = static_cast<uint16_t>(raw[k] & 0xffffu);
+                    v[2 * k + 1] = static_cast<uint16_t>(raw[k] >> 16);
                 }
             } else {
 #pragma unroll
@@ -276,29 +288,32 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
             for (int k = 0; k < 8; ++k)
                 if (gc + k < d.cols) v[k] = f2bf(bf2f(v[k]) / den);
         }
-        uint4 o;
-        o.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
-        o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
-        o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
-        o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
-        *reinterpret_cast<uint4*>(d.direct + static_cast<int64_t>(gr) * d.ld_direct + gc) = o;
+        u32x4e o;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) tile[r][cc + k] = v[k];
+        for (int k = 0; k < 4; ++k) o[k] = v[2 * k] | (static_cast<uint32_t>(v[2 * k + 1]) << 16);
+        gst4u(d.direct + static_cast<int64_t>(gr) * d.ld_direct + gc, o);
+        uint2* const dst = reinterpret_cast<uint2*>(&tile[r][cc / 2]);
+        dst[0] = make_uint2(o[0], o[1]);
+        dst[1] = make_uint2(o[2], o[3]);
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < (NT_TILE / 2) * CH / 256; ++i) {
+        // work item -> word column c (transposed rows 2c, 2c+1) and source rows r0 .. r0+7
         const int q = threadIdx.x + i * 256;
-        const int tr = q >> 3, tc = (q & 7) * 8;   // transposed tile: row tr (a source column)
-        uint16_t v[8];
+        const int c = q / CH, r0 = (q % CH) * 8;
+        uint32_t w[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = tile[tc + k][tr];
-        uint4 o;
-        o.x = v[0] | (static_cast<uint32_t>(v[1]) << 16);
-        o.y = v[2] | (static_cast<uint32_t>(v[3]) << 16);
-        o.z = v[4] | (static_cast<uint32_t>(v[5]) << 16);
-        o.w = v[6] | (static_cast<uint32_t>(v[7]) << 16);
-        *reinterpret_cast<uint4*>(d.transp + static_cast<int64_t>(C0 + tr) * d.ld_transp + R0 + tc) = o;
+        for (int k = 0; k < 8; ++k) w[k] = tile[r0 + k][c];
+        u32x4e lo, hi;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            lo[k] = (w[2 * k] & 0xffffu) | (w[2 * k + 1] << 16);
+            hi[k] = (w[2 * k] >> 16) | (w[2 * k + 1] & 0xffff0000u);
+        }
+        uint16_t* const t = d.transp + static_cast<int64_t>(C0 + 2 * c) * d.ld_transp + R0 + r0;
+        gst4u(t, lo);
+        gst4u(t + d.ld_transp, hi);
     }
 }
 

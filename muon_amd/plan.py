@@ -32,7 +32,7 @@ SUPER_DIMS = {0: (8, 8), 1: (4, 8)}
 if os.environ.get("MUON_AMD_SUPER"):     # measurement knob: "rows,cols" of the 256 x 256 class super-block
     SUPER_DIMS[1] = tuple(int(v) for v in os.environ["MUON_AMD_SUPER"].split(","))
 EW_BLOCK_ELEMS = 8192                   # must match muon_amd_elementwise_block_elems()
-NT_TILE = 64                            # must match muon_amd_normalize_tile()
+NT_TILE = 128                           # must match muon_amd_normalize_tile()
 N_XCD = 8                               # workgroups are dealt round-robin to the 8 XCDs
 # Workspace rows may be made this many elements longer than the padded width (a knob for
 # measurements: on MI355X a power-of-two row pitch measured no slower than a padded one).
