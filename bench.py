@@ -143,6 +143,37 @@ def summarize_kernels(per_label):
     return out, gemm_work, gemm_ms, gemm_n
 
 
+def run_ns32(steps, warmup, seed):
+    """Benchmark configuration 3: 32 independent 4096 x 4096 bf16 matrices ~N(0,1) through
+    zeropower_via_newtonschulz5 (5 iterations); one call is one step."""
+    import muon_amd
+    from muon_amd import engine
+
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(seed)
+    G = torch.randn(32, 4096, 4096, device="cuda:0", generator=gen).bfloat16()
+    for _ in range(warmup):
+        muon_amd.zeropower_via_newtonschulz5(G)
+    torch.cuda.synchronize()
+    engine.PROFILE = []
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = muon_amd.zeropower_via_newtonschulz5(G)
+    torch.cuda.synchronize()
+    total_ms = (time.perf_counter() - t0) * 1e3
+    prof, engine.PROFILE = engine.PROFILE, None
+    assert torch.isfinite(out[0]).all()
+    per_label = {}
+    for label, work, e0, e1 in prof:
+        d = per_label.setdefault(label, [0.0, 0.0, 0])
+        d[0] += work
+        d[1] += e0.elapsed_time(e1)
+        d[2] += 1
+    muon_amd.clear_engine_cache()
+    return dict(ms_per_step=total_ms / steps, per_label=per_label, muon_elements=32 * 4096 * 4096, adam_elements=0,
+                f_sym=32 * f_sym(4096, 4096), f_dense=32 * f_dense(4096, 4096))
+
+
 # ------------------------------------------------------------------------------------------
 # CPU baseline: the oracle restatement of the reference on the host cores, bounded sample
 # ------------------------------------------------------------------------------------------
@@ -195,7 +226,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="llama3-8b", choices=["llama3-8b", "gpt2-124m", "conv"])
+    ap.add_argument("--workload", default="llama3-8b", choices=["llama3-8b", "gpt2-124m", "conv", "ns32"])
     ap.add_argument("--ns-variant", default="ns5", choices=["ns5", "aol4"],
                     help="ns5: the five-iteration specification (the headline); aol4: the 4-iteration "
                          "AOL-rescaled variant (its flop count is 11/15 of the headline's, so only the step "
@@ -214,6 +245,27 @@ def main():
                  "by matrix across ranks, which is not part of this library). Run with --gpus 1.")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X GPU")
+    if args.workload == "ns32":
+        steps = args.steps if args.steps is not None else 5
+        warmup = args.warmup if args.warmup is not None else 1
+        res = run_ns32(steps, warmup, seed=1234 + 3)
+        kernels, gemm_work, gemm_ms, gemm_n = summarize_kernels(res["per_label"])
+        print(json.dumps({
+            "metric": "ns5_ms_32x4096x4096_bf16", "value": round(res["ms_per_step"], 3), "unit": "ms", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(res["ms_per_step"], 3),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "ns32: zeropower_via_newtonschulz5 on 32 x 4096 x 4096 bf16 ~N(0,1), 5 iterations",
+                       "rounding": "reference"},
+            "roofline": {"bound": "mfma", "kernel": "ns_gemm_kernel (syrk + poly + update launches)",
+                         "achieved": round(gemm_work / gemm_ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(gemm_work / gemm_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                         "launches": gemm_n, "avg_launch_ms": round(gemm_ms / gemm_n, 4),
+                         "flops_per_launch": gemm_work / gemm_n},
+            "ns": {"tflops_sym_whole_call": round(res["f_sym"] / res["ms_per_step"] / 1e9, 1),
+                   "tflops_dense_equiv_whole_call": round(res["f_dense"] / res["ms_per_step"] / 1e9, 1)},
+            "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kernels.items()},
+        }))
+        return
     _, _, _, dsteps, dwarm = workload_shapes(args.workload)
     steps = args.steps if args.steps is not None else dsteps
     warmup = args.warmup if args.warmup is not None else dwarm

@@ -121,6 +121,7 @@ class _ChunkRuntime:
         self.mat_dev = _upload(d, self.device, into=self.mat_dev)
         self.mat_key = key
         self.src_dtypes = list(src_dtypes)
+        self.present = [(bool(m), bool(p), bool(o)) for m, p, o in zip(momenta, params, outs)]
 
     def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor, scalars_ptr=0):
         """Enqueue the chunk's launches.  scalars_ptr: device address of {one_minus_beta, beta, lr,
@@ -137,8 +138,10 @@ class _ChunkRuntime:
         # algorithmic bytes: gradient, momentum (read + write) and parameter (read + write) in
         # their storage type, the bf16 update written once and read once
         store = [2 if t == _lib.SRC_BF16 else 4 for t in self.src_dtypes]
-        mom_bytes = sum(lay.numel * (3 * sz + 2) for lay, sz in zip(c.layouts, store))
-        apply_bytes = sum(lay.numel * (2 * sz + 2) for lay, sz in zip(c.layouts, store))
+        mom_bytes = sum(lay.numel * (sz + 2 + (2 * sz if has_m else 0))
+                        for lay, sz, (has_m, _, _) in zip(c.layouts, store, self.present))
+        apply_bytes = sum(lay.numel * (2 + (2 * sz if has_p else 0) + (2 if has_o else 0))
+                          for lay, sz, (_, has_p, has_o) in zip(c.layouts, store, self.present))
         _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
             int(mutate_grad), sc_mom, s), "momentum"))
