@@ -1,4 +1,4 @@
-"""Writes tests/golden/ns_golden.npz and tests/golden/step_golden.npz from the CPU oracle.
+"""Writes tests/golden/ns_golden.npz, step_golden.npz and aol4_golden.npz from the CPU oracle.
 
 The reference ships no golden vectors and its Newton-Schulz contract (muon.py:265-291) is
 comment text, so these fixtures come from oracle/muon_oracle.py, whose functions are pinned by
@@ -23,7 +23,22 @@ def bf16_bits(t):
     return t.contiguous().view(torch.int16).numpy().astype(np.uint16)
 
 
+def aol4():
+    """Fixtures of the 4-iteration AOL-rescaled variant (oracle.ns_aol4, pinned by its SVD closed form)."""
+    torch.manual_seed(20251126)
+    out = {}
+    for name, shape, std in [("wide_16x48", (16, 48), 1e-3), ("tall_48x16", (48, 16), 1e-3),
+                             ("square_24x24", (24, 24), 1.0), ("wide_40x136", (40, 136), 1e-2),
+                             ("batched_3x12x20", (3, 12, 20), 1.0)]:
+        G = torch.randn(*shape) * std * (torch.rand(*shape[:-1], 1) * 3 + 0.05)
+        out[name + "/in"] = G.numpy()
+        out[name + "/bf16"] = bf16_bits(O.ns_aol4(G))
+        out[name + "/fp64_closed_form"] = O.ns_aol4_closed_form(G.bfloat16().double().numpy())
+    np.savez_compressed(os.path.join(HERE, "aol4_golden.npz"), **out)
+
+
 def main():
+    aol4()
     torch.manual_seed(20251125)
     ns = {}
     for name, shape, std in [("wide_16x48", (16, 48), 1e-3), ("tall_48x16", (48, 16), 1e-3),

@@ -621,3 +621,31 @@ def test_split_reduction_is_deterministic_and_batch_independent(M):
     got = M.zeropower_via_newtonschulz5(_dev(wide))
     assert torch.equal(got, M.zeropower_via_newtonschulz5(_dev(wide)))
     assert O.rel_fro(got.float().cpu(), O.ns5_bf16(wide).float()) <= TOL_BF16
+
+
+def test_aol4_golden_fixtures(M, golden_dir):
+    z = np.load(os.path.join(golden_dir, "aol4_golden.npz"))
+    for name in sorted({k.split("/")[0] for k in z.files}):
+        got = M.zeropower_via_aol4(_dev(torch.from_numpy(z[name + "/in"]))).float().cpu()
+        want = torch.from_numpy(z[name + "/bf16"].astype(np.int16)).view(torch.bfloat16).float()
+        assert O.rel_fro(got, want) <= TOL_BF16, name
+        assert O.rel_fro(got.double(), z[name + "/fp64_closed_form"]) <= TOL_FP32, name
+
+
+def test_graph_replay_with_aol4_and_bf16_storage(M):
+    """The opt-in paths compose: graph replay of the AOL variant on bf16 parameters equals eager."""
+    torch.manual_seed(1350)
+    base = [(torch.randn(*s) * 0.02).bfloat16() for s in [(256, 384), (128, 2048), (2, 64, 96)]]
+    pe = [torch.nn.Parameter(_dev(b.clone())) for b in base]
+    pg = [torch.nn.Parameter(_dev(b.clone())) for b in base]
+    oe = M.SingleDeviceMuon(pe, lr=0.02, weight_decay=0.01, ns_variant="aol4")
+    og = M.SingleDeviceMuon(pg, lr=0.02, weight_decay=0.01, ns_variant="aol4", use_graph=True)
+    for step in range(3):
+        for a, b in zip(pe, pg):
+            g = (torch.randn(*a.shape, device="cuda") * 1e-2).bfloat16()
+            a.grad, b.grad = g.clone(), g.clone()
+        oe.step()
+        og.step()
+        torch.cuda.synchronize()
+        for a, b in zip(pe, pg):
+            assert torch.equal(a.detach(), b.detach()), step

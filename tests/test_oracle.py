@@ -319,3 +319,13 @@ def test_row_only_rescaling_of_the_gram_matrix_is_not_a_contraction():
     G = _uneven_rows((30, 200), 3)
     assert rows_only(G, True) > 10 and rows_only(G, False) > 10
     assert torch.linalg.svdvals(O.ns_aol4(G, work_dtype=torch.float64)).max() < 1.25
+
+
+def test_aol4_golden_fixture_is_what_the_oracle_computes(golden_dir):
+    z = np.load(os.path.join(golden_dir, "aol4_golden.npz"))
+    for name in sorted({k.split("/")[0] for k in z.files}):
+        G = torch.from_numpy(z[name + "/in"])
+        got = O.ns_aol4(G)
+        want = torch.from_numpy(z[name + "/bf16"].astype(np.int16)).view(torch.bfloat16)
+        assert O.rel_fro(got.float(), want.float()) < 1e-6, name        # bf16 CPU matmuls are deterministic here
+        assert O.rel_fro(got.double(), z[name + "/fp64_closed_form"]) < 2e-2, name
