@@ -256,10 +256,12 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 // ---------------------------------------------------------------------------------------------
 // The LDS ring holds NHALF half-stages; a half-stage is the P rows or the Q rows of one k-block
 // (BT rows x 128 bytes).  Half-stages are issued in the order P0 Q0 P1 Q1 P2 ...; block kb needs
-// halves 2kb and 2kb+1.  While block kb is multiplied, the halves up to 2kb+NHALF-3 (issued in
-// earlier iterations) and halves 2kb+NHALF-2, 2kb+NHALF-1 (issued during this iteration into the
-// two slots block kb-1 vacated) are in flight, so the load pipe always has queued requests and
-// every request is a full 128-byte line.  NHALF = 5 fills the 160 KB LDS for the 256 x 256 tile.
+// halves 2kb and 2kb+1.  The prologue issues the first NHALF; the pair 2kb+NHALF, 2kb+NHALF+1 goes
+// into the two slots of block kb, from the last k-step of block kb (every fragment of the block is
+// in registers by then) through the first three k-steps of block kb+1.  So while a block is
+// multiplied the next one and a half are in flight or landed, the load pipe always has queued
+// requests, and every request is a full 128-byte line.  NHALF = 5 fills the 160 KB LDS for the
+// 256 x 256 tile.
 template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_, bool SPLIT_K_>
 struct GemmCfg {
     static constexpr bool SPLIT_K = SPLIT_K_;     // jobs may share a tile's reduction
