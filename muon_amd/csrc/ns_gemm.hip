@@ -43,8 +43,14 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ u32x2 gload8(const uint16_t* p) {
     return *(const __attribute__((address_space(1))) u32x2*)(p);
 }
+// STREAM: non-temporal hint.  The outputs of the large tile class are hundreds of megabytes that
+// the next launch reads long after this XCD's L2 has turned over; keeping them out of the way of
+// the operand panels measured +0.5 % on the Llama step (and a loss for GPT-2-size matrices, whose
+// outputs the next launch does find in L2, so the small class stores normally).
+template <bool STREAM>
 __device__ __forceinline__ void gstore16(uint16_t* p, u32x4 v) {
-    *(__attribute__((address_space(1))) u32x4*)(p) = v;
+    if constexpr (STREAM) __builtin_nontemporal_store(v, (__attribute__((address_space(1))) u32x4*)(p));
+    else *(__attribute__((address_space(1))) u32x4*)(p) = v;
 }
 
 constexpr int BK = 64;   // k extent of one ring stage (128 bytes per LDS row)
@@ -117,7 +123,7 @@ constexpr int epilogue_stage_bytes(int WM, int WN) {
 // Per 32 x 32 tile: t1 = alpha*acc -> row-owning layout -> + beta*D (8-byte loads) -> o (bf16)
 // -> staged row-major in LDS -> 16-byte coalesced stores of C (and gamma*o to C2); o moved back
 // to the column-owning layout -> staged -> 16-byte coalesced stores of CT (and C2T).
-template <bool HAS_D, int WGN, int WM, int WN, int TM, int TN>
+template <bool HAS_D, bool STREAM, int WGN, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const MuonGemmDesc& d,
                                                  const MuonTileJob& job, float alpha, float beta,
                                                  float gamma, bool round_terms, char* stage) {
@@ -219,8 +225,8 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
             if (r < RPI && row < WM) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
                 const size_t off = static_cast<size_t>(row0 + row) * d.ldc + col0 + ch * 8;
-                gstore16(d.C + off, v);
-                if (d.C2) gstore16(d.C2 + off, scale_bf16x8(v, gamma));
+                gstore16<STREAM>(d.C + off, v);
+                if (d.C2) gstore16<STREAM>(d.C2 + off, scale_bf16x8(v, gamma));
             }
         }
     }
@@ -244,8 +250,8 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
             if (r < RPI && row < WN) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
                 const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + ch * 8;
-                gstore16(d.CT + off, v);
-                if (d.C2T) gstore16(d.C2T + off, scale_bf16x8(v, gamma));
+                gstore16<STREAM>(d.CT + off, v);
+                if (d.C2T) gstore16<STREAM>(d.C2T + off, scale_bf16x8(v, gamma));
             }
         }
     }
@@ -265,6 +271,7 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_, bool SPLIT_K_>
 struct GemmCfg {
     static constexpr bool SPLIT_K = SPLIT_K_;     // jobs may share a tile's reduction
+    static constexpr bool STREAM_STORES = BT_ >= 256;   // see gstore16
     static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_, NHALF = NHALF_;
     static constexpr int NW = WGM * WGN, NT = NW * 64;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
@@ -494,8 +501,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     }
     char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
     const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
-    if (d.D) ns_epilogue_impl<true, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
-    else ns_epilogue_impl<false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
+    if (d.D) ns_epilogue_impl<true, Cfg::STREAM_STORES, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
+    else ns_epilogue_impl<false, Cfg::STREAM_STORES, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
 }
 
 // Tile classes: square output tile, waves, workgroups per CU.
