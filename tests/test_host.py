@@ -280,3 +280,32 @@ def test_aol_variant_plan_validates():
         assert lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix), _lib.host_ptr(bad)) == -1
     ns5 = plan.plan_chunks(SHAPES, 5, True, 1 << 30)
     assert all(a.workspace_bytes > b.workspace_bytes for a, b in zip(chunks, ns5))
+
+
+def test_header_is_plain_c_and_field_offsets_match_the_binding(tmp_path):
+    """include/muon_amd.h compiles as C99 on its own, and every struct field sits where the numpy
+    mirror of the binding puts it."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    structs = {"MuonMatDesc": _lib.MAT_DESC, "MuonGemmDesc": _lib.GEMM_DESC, "MuonTileJob": _lib.TILE_JOB,
+               "MuonAdamDesc": _lib.ADAM_DESC, "MuonAolDesc": _lib.AOL_DESC}
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "muon_amd.h"', 'int main(void) {']
+    for name, dt in structs.items():
+        lines.append(f'  printf("{name} size %zu\\n", sizeof({name}));')
+        for field in dt.names:
+            lines.append(f'  printf("{name} {field} %zu\\n", offsetof({name}, {field}));')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "offsets.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "offsets"
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-I", inc, str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    got = {tuple(l.split()[:2]): int(l.split()[2]) for l in out if l}
+    for name, dt in structs.items():
+        assert got[(name, "size")] == dt.itemsize
+        for field in dt.names:
+            assert got[(name, field)] == dt.fields[field][1], (name, field)
