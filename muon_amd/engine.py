@@ -65,7 +65,8 @@ class _ChunkRuntime:
                                                   chunk.split_slots if ph == _plan.PH_SYRK else 0),
                        "validate_gemm")
         self.mat_template = chunk.mat_descs(base)
-        # one static device blob: gemm descs | sym jobs | full jobs | block prefix | tile prefix
+        # one static device blob: gemm descs | sym jobs | full jobs | block prefix | tile prefix |
+        # syrk jobs (| AOL descs | AOL row prefix | AOL segment prefix), each part 256-byte aligned
         parts = [gemm.reshape(-1).view(np.uint8), chunk.sym_jobs.view(np.uint8),
                  chunk.full_jobs.view(np.uint8), chunk.block_prefix.view(np.uint8),
                  chunk.tile_prefix.view(np.uint8), chunk.syrk_jobs.view(np.uint8)]
