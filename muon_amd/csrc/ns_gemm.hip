@@ -144,19 +144,39 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
         id1[t] = static_cast<__bf16>(16 + rho == lr ? 1.0f : 0.0f);
     }
 
-    // addend: lane owns row (a*32 + lr) and columns b*32 + 8q + 4g .. +4 -> one 8-byte load each,
-    // all issued before the first is used.  D may alias C (in-place a*X + B*X): every load of
-    // this wave's sub-tile precedes its stores through the data dependence on o.
+    // addend: the lane that owns row (a*32 + lr) needs columns b*32 + 8q + 4g .. +4 of it.  Fetched
+    // that way from global memory, every load instruction would touch 32 different rows for 16
+    // bytes each and the address pipe would take longer than the whole rest of the epilogue.  So
+    // the wave's WM x 64 piece of D is first streamed into its staging area by the DMA path, one
+    // instruction per 8 full rows (chunks XOR-swizzled as in the operand ring), and the
+    // row-owning 8-byte pieces are read from LDS.  All of them are in registers before the
+    // staging area is reused for the results, and before any store of this sub-tile (D may alias
+    // C: in-place a*X + B*X).
+    static_assert(WN == 64, "the addend staging assumes 128-byte rows");
     u32x2 dv[TM][TN][4];
     if (HAS_D) {
+        const uint32_t stage_lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(
+            reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)stage)));
+        const int drow = lane >> 3;                         // row within the 8 rows of one instruction
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+        for (int j = 0; j < WM / 8; ++j) {
+            const int rr = j * 8 + drow;
+            const int lc = (lane & 7) ^ ((rr >> 1) & 7);    // logical 16-byte chunk this lane fetches
+            dma16(d.D + static_cast<size_t>(row0 + rr) * d.ldd + col0 + lc * 8, stage_lds + j * 1024);
+        }
+        NS_WAIT_VMCNT(0);
+#pragma unroll
+        for (int a = 0; a < TM; ++a) {
+            const int rr = a * 32 + lr;
 #pragma unroll
             for (int b = 0; b < TN; ++b)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    dv[a][b][q] = gload8(d.D + static_cast<size_t>(row0 + a * 32 + lr) * d.ldd + col0 +
-                                         b * 32 + 8 * q + 4 * g);
+                    dv[a][b][q] = *reinterpret_cast<const u32x2*>(
+                        stage + rr * 128 + (((b * 4 + q) ^ ((rr >> 1) & 7)) * 16) + g * 8);
+        }
+        // (a wave's LDS operations execute in order: these reads are done before the results
+        // below overwrite the area)
     }
 
     uint32_t ot[TM][TN][8];   // results moved back to accumulator layout, packed bf16 pairs
@@ -595,14 +615,14 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJ
                      "gemm desc %d: output %dx%d is not in tiles of %dx%d", i, d.rows, d.colsn, TR, TC);
         MUON_REQUIRE(d.ldp >= d.K && d.ldq >= d.K && d.ldp % 8 == 0 && d.ldq % 8 == 0,
                      "gemm desc %d: ldp=%d ldq=%d K=%d", i, d.ldp, d.ldq, d.K);
-        MUON_REQUIRE(!d.D || (d.ldd >= d.colsn && d.ldd % 4 == 0), "gemm desc %d: ldd=%d cols %d", i, d.ldd, d.colsn);
+        MUON_REQUIRE(!d.D || (d.ldd >= d.colsn && d.ldd % 8 == 0), "gemm desc %d: ldd=%d cols %d", i, d.ldd, d.colsn);
         MUON_REQUIRE(!(d.C || d.C2) || (d.ldc >= d.colsn && d.ldc % 8 == 0), "gemm desc %d: ldc=%d cols %d", i, d.ldc, d.colsn);
         MUON_REQUIRE(!(d.CT || d.C2T) || (d.ldct >= d.rows && d.ldct % 8 == 0),
                      "gemm desc %d: ldct=%d rows=%d", i, d.ldct, d.rows);
         MUON_REQUIRE((reinterpret_cast<uintptr_t>(d.P) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.Q) % 16) == 0 &&
                          (reinterpret_cast<uintptr_t>(d.C) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.C2) % 16) == 0 &&
                          (reinterpret_cast<uintptr_t>(d.CT) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.C2T) % 16) == 0 &&
-                         (reinterpret_cast<uintptr_t>(d.D) % 8) == 0,
+                         (reinterpret_cast<uintptr_t>(d.D) % 16) == 0,
                      "gemm desc %d: misaligned pointer", i);
         MUON_REQUIRE(!(d.C2 && !d.C) && !(d.C2T && !d.CT), "gemm desc %d: scaled copy needs its primary output", i);
     }
