@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM-side bytes per ns_gemm launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this
 # script, scaled by what the counters read for a 1 GiB copy; averaged over the launches of a step)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 1.898e10}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 1.950e10}
 
 
 # ------------------------------------------------------------------------------------------
