@@ -649,3 +649,20 @@ def test_graph_replay_with_aol4_and_bf16_storage(M):
         torch.cuda.synchronize()
         for a, b in zip(pe, pg):
             assert torch.equal(a.detach(), b.detach()), step
+
+
+def test_llama_layer_shapes_one_step(M):
+    """One full step on the matrix shapes of a Llama-3-8B layer (the 256 x 256 tile class at its
+    real sizes: wide, tall and the 1024-row k/v projection) against the oracle."""
+    shapes = [(4096, 14336), (14336, 4096), (1024, 4096), (4096, 4096)]
+    cpu, gpu = _clone_params(shapes, 0.02, 1360)
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    _set_grads(cpu, gpu, 1e-4)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    oc.step()
+    og.step()
+    for pc, pg in zip(cpu, gpu):
+        assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= TOL_PARAM, tuple(pc.shape)
+        np.testing.assert_allclose(og.state[pg]["momentum_buffer"].cpu().numpy(),
+                                   oc.state[pc]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-12)
