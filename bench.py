@@ -5,10 +5,14 @@
 
 A step is one full SingleDeviceMuonWithAuxAdam.step() over the synthetic parameter set of the
 workload (seeded random parameters and gradients resident in HBM before the timed region starts;
-the K timed steps run back to back between two device synchronisations).  Prints
-one JSON line: step time, the MFMA roofline of the Newton-Schulz GEMM launches measured with HIP
-events on the launch stream, the HBM fractions of the elementwise kernels, and the CPU baseline
-(the oracle restatement of the reference timed on the host cores over a bounded sample).
+the K timed steps run back to back between two device synchronisations).  Before anything is timed
+the HIP path is checked against the CPU oracle on the shapes of the workload (Newton-Schulz within
+2e-2 of the bf16 restatement and 3e-2 of fp32, parameters within 1e-3 after a step, Adam within
+1e-5); a failed gate ends the run with a non-zero exit code and no JSON line.  Prints one JSON
+line: step time, the MFMA roofline of the Newton-Schulz GEMM launches measured with HIP events on
+the launch stream, the HBM fractions of the elementwise kernels, the other benchmark configurations
+as sub-objects, and the CPU baseline (the oracle restatement of the reference timed on the host
+cores over a bounded sample).
 """
 from __future__ import annotations
 
@@ -25,9 +29,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
-# HBM-side bytes per ns_gemm launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this
-# script, scaled by what the counters read for a 1 GiB copy; averaged over the launches of a step)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": 1.950e10}
+# HBM-side bytes per ns_gemm launch: NOT measured by this script.  The figure comes from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE, scaled by what the counters read for
+# a 1 GiB copy, averaged over the launches of a step); the summary file is named beside it.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": (1.950e10, "profiles/hbm_traffic_llama3-8b_step.md")}
+
+TOL_NS_BF16, TOL_NS_FP32, TOL_PARAM, TOL_ADAM = 2e-2, 3e-2, 1e-3, 1e-5
 
 
 # ------------------------------------------------------------------------------------------
@@ -68,9 +75,76 @@ def mat2d(shape):
 
 
 # ------------------------------------------------------------------------------------------
+# correctness gates (run before anything is timed)
+# ------------------------------------------------------------------------------------------
+def correctness_gates(name):
+    """The HIP path against the CPU oracle on one instance of every distinct Muon shape of the
+    workload (Newton-Schulz output and one optimizer step) and on a slab of every Adam shape.
+    Returns the measured distances; ends the run when one exceeds its bound."""
+    import muon_amd
+    from oracle import muon_oracle as O
+
+    torch.set_num_threads(host_threads())
+    res, failed = {}, []
+
+    def gate(key, value, bound):
+        res[key] = round(float(value), 6)
+        if not value <= bound:
+            failed.append(f"{key} = {value:.3e} > {bound:.3e}")
+
+    torch.manual_seed(97)
+    if name == "ns32":
+        G = torch.randn(4096, 4096).bfloat16()
+        got = muon_amd.zeropower_via_newtonschulz5(G.cuda()).float().cpu()
+        ref16, ref32 = O.ns5_bf16(G).float(), O.ns5_fp32(G.float())
+        gate("ns_vs_bf16_4096x4096", O.rel_fro(got, ref16), TOL_NS_BF16)
+        gate("ns_vs_fp32_4096x4096", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+    else:
+        muon, adam, gstd, _, _ = workload_shapes(name)
+        for shape, _ in muon:
+            tag = "x".join(str(v) for v in shape)
+            p_c = torch.nn.Parameter(torch.randn(*shape) * 0.02)
+            p_g = torch.nn.Parameter(p_c.detach().clone().cuda())
+            g = torch.randn(*shape) * gstd
+            p_c.grad, p_g.grad = g.clone(), g.clone().cuda()
+            g2 = g.reshape(mat2d(shape))
+            got = muon_amd.zeropower_via_newtonschulz5(g2.cuda()).float().cpu()
+            ref16, ref32 = O.ns5_bf16(g2).float(), O.ns5_fp32(g2)
+            gate(f"ns_vs_bf16_{tag}", O.rel_fro(got, ref16), TOL_NS_BF16)
+            # where the reference's own bf16 result is further than 3e-2 from fp32 (small conv
+            # shapes), the kernel that follows its rounding sequence inherits that distance
+            gate(f"ns_vs_fp32_{tag}", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+            O.OracleSingleDeviceMuon([p_c], lr=0.02, weight_decay=0.01, momentum=0.95).step()
+            muon_amd.SingleDeviceMuon([p_g], lr=0.02, weight_decay=0.01, momentum=0.95).step()
+            # a tiny filter's update is several per cent of |p|, so bf16 Newton-Schulz noise weighs more there
+            gate(f"param_after_step_{tag}", O.rel_fro(p_g.detach().cpu(), p_c.detach()),
+                 TOL_PARAM if min(mat2d(shape)) >= 128 else 3e-3)
+        for shape, _ in adam:
+            sl = (min(shape[0], 4096),) + tuple(shape[1:])
+            tag = "x".join(str(v) for v in sl)
+            p_c = torch.nn.Parameter(torch.randn(*sl) * 0.02)
+            p_g = torch.nn.Parameter(p_c.detach().clone().cuda())
+            kw = dict(use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)
+            oc = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p_c], **kw)])
+            og = muon_amd.SingleDeviceMuonWithAuxAdam([dict(params=[p_g], **kw)])
+            for _ in range(2):
+                g = torch.randn(*sl) * gstd
+                p_c.grad, p_g.grad = g.clone(), g.clone().cuda()
+                oc.step()
+                og.step()
+            d = (p_g.detach().cpu() - p_c.detach()).abs() / p_c.detach().abs().clamp_min(1e-3)
+            gate(f"adam_max_rel_{tag}", d.max(), TOL_ADAM)
+    muon_amd.clear_engine_cache()
+    torch.cuda.empty_cache()
+    if failed:
+        sys.exit("bench.py: correctness gate failed before timing: " + "; ".join(failed))
+    return res
+
+
+# ------------------------------------------------------------------------------------------
 # GPU leg
 # ------------------------------------------------------------------------------------------
-def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False):
+def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False, realloc_grads=False):
     import muon_amd
     from muon_amd import engine
 
@@ -97,8 +171,20 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_grap
     # momentum and the parameters move every step, so every step orthogonalises new matrices.
     for p in pm + pa:
         p.grad.normal_(0.0, gstd, generator=gen)
-    for _ in range(warmup):
+    # --realloc-grads: what a training loop with zero_grad(set_to_none=True) does to the optimizer.
+    # Every gradient sits at another address than the step before, so the descriptor tables are
+    # re-validated and uploaded again inside the timed region.  Two resident sets alternate, so no
+    # copy or allocation of the gradients themselves is timed.
+    spare = [p.grad.clone() for p in pm + pa] if realloc_grads else None
+
+    def one_step():
+        if spare is not None:
+            for i, p in enumerate(pm + pa):
+                p.grad, spare[i] = spare[i], p.grad
         opt.step()
+
+    for _ in range(warmup):
+        one_step()
     torch.cuda.synchronize()
 
     # timed region: exactly `steps` steps back to back, one synchronisation on either side; a pair
@@ -106,7 +192,7 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_grap
     engine.PROFILE = None if use_graph else []      # a replayed graph has no per-launch events
     t0 = time.perf_counter()
     for _ in range(steps):
-        opt.step()
+        one_step()
     torch.cuda.synchronize()
     total_ms = (time.perf_counter() - t0) * 1e3
     prof, engine.PROFILE = engine.PROFILE or [], None
@@ -121,9 +207,8 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_grap
     n_a = sum(p.numel() for p in pa)
     fs = sum(f_sym(min(mat2d(s)), max(mat2d(s))) * c for s, c in muon)
     fd = sum(f_dense(min(mat2d(s)), max(mat2d(s))) * c for s, c in muon)
-    # sanity: the state after the timed steps is finite
     assert all(torch.isfinite(p).all() for p in pm[:2] + pa[:2])
-    del opt, pm, pa
+    del opt, pm, pa, spare
     torch.cuda.empty_cache()
     return dict(ms_per_step=total_ms / steps, per_label=per_label, muon_elements=n_m, adam_elements=n_a,
                 f_sym=fs, f_dense=fd)
@@ -169,21 +254,95 @@ def run_ns32(steps, warmup, seed):
         d[0] += work
         d[1] += e0.elapsed_time(e1)
         d[2] += 1
+    del out, G
     muon_amd.clear_engine_cache()
+    torch.cuda.empty_cache()
     return dict(ms_per_step=total_ms / steps, per_label=per_label, muon_elements=32 * 4096 * 4096, adam_elements=0,
                 f_sym=32 * f_sym(4096, 4096), f_dense=32 * f_dense(4096, 4096))
+
+
+def roofline_object(workload, gemm_work, gemm_ms, gemm_n):
+    traffic = GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(workload)
+    return {
+        "bound": "mfma",
+        "kernel": "ns_gemm_kernel (syrk + poly + update launches)",
+        "achieved": round(gemm_work / gemm_ms / 1e9, 1),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(gemm_work / gemm_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+        "traffic": traffic[0] if traffic else None,
+        "traffic_source": (traffic[1] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this "
+                           "command; a profile-derived constant, not measured in this run)") if traffic else None,
+        "launches": gemm_n,
+        "avg_launch_ms": round(gemm_ms / gemm_n, 4),
+        "flops_per_launch": gemm_work / gemm_n,
+    }
+
+
+def rounded(kernels):
+    return {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kernels.items()}
+
+
+SECONDARY_SEEDS = {"gpt2-124m": 1234 + 2, "conv": 1234 + 5}
+
+
+def secondary(name, gates):
+    """A further benchmark configuration measured in the same run, as a sub-object."""
+    out = {"gates": correctness_gates(name)} if gates else {}
+    if name == "ns32":
+        r = run_ns32(3, 1, seed=1234 + 3)
+    else:
+        _, _, _, dsteps, dwarm = workload_shapes(name)
+        r = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name])
+    _, gw, gms, gn = summarize_kernels(r["per_label"])
+    out.update({"ms_per_step": round(r["ms_per_step"], 3), "ns_tflops_sym": round(gw / gms / 1e9, 1),
+                "ns_frac_of_peak": round(gw / gms / 1e9 / PEAK_BF16_TFLOPS, 4), "gemm_launches": gn,
+                "avg_gemm_launch_ms": round(gms / gn, 4)})
+    if name != "ns32":
+        g = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], use_graph=True)
+        out["ms_per_step_graph_replay"] = round(g["ms_per_step"], 3)
+    return out
 
 
 # ------------------------------------------------------------------------------------------
 # CPU baseline: the oracle restatement of the reference on the host cores, bounded sample
 # ------------------------------------------------------------------------------------------
+def host_threads():
+    """Threads for the host-side legs: every core the process may use (bounded by the
+    OMP_NUM_THREADS of the environment when that is set, as on a host whose cores are shared)."""
+    n = os.cpu_count() or 1
+    if hasattr(os, "sched_getaffinity"):
+        n = min(n, len(os.sched_getaffinity(0)))
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    if env.isdigit() and int(env) > 0:
+        n = min(n, int(env))
+    return n
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(name, budget_s=25.0):
     from oracle import muon_oracle as O
-    cores = min(16, os.cpu_count() or 1)
+    cores = host_threads()
     torch.set_num_threads(cores)
     muon, adam, gstd, _, _ = workload_shapes(name)
     torch.manual_seed(4321)
     total_ms, parts, t_start = 0.0, [], time.perf_counter()
+
+    def timed_step(opt):
+        opt.step()                      # warm-up: thread pool, allocator, lazy state
+        t0 = time.perf_counter()
+        opt.step()
+        return (time.perf_counter() - t0) * 1e3
+
     # one instance of each distinct Muon shape; a shape and its transpose cost the same (the
     # iteration runs on the wide orientation either way), so they share one timing
     merged = {}
@@ -197,26 +356,22 @@ def cpu_baseline(name, budget_s=25.0):
             continue
         p = torch.nn.Parameter(torch.randn(*shape) * 0.02)
         p.grad = torch.randn(*shape) * gstd
-        opt = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=True, lr=0.02, weight_decay=0.01)])
-        t0 = time.perf_counter()
-        opt.step()
-        ms = (time.perf_counter() - t0) * 1e3
+        ms = timed_step(O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=True, lr=0.02, weight_decay=0.01)]))
         total_ms += ms * count
-        parts.append(f"{count}x{tuple(shape)}@{ms:.0f}ms")
+        parts.append(f"muon {count}x{tuple(shape)}@{ms:.0f}ms")
     # Adam: one slab of at most 4096 rows of each distinct shape, scaled by element count
     for shape, count in adam:
         rows = min(shape[0], 4096)
         sl = (rows,) + tuple(shape[1:])
         p = torch.nn.Parameter(torch.randn(*sl) * 0.02)
         p.grad = torch.randn(*sl) * gstd
-        opt = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=False, weight_decay=0.01)])
-        t0 = time.perf_counter()
-        opt.step()
-        ms = (time.perf_counter() - t0) * 1e3 * (shape[0] / rows)
+        ms = timed_step(O.OracleSingleDeviceMuonWithAuxAdam([dict(params=[p], use_muon=False, weight_decay=0.01)]))
+        ms *= shape[0] / rows
         total_ms += ms * count
+        parts.append(f"adam {count}x{tuple(shape)}@{ms:.1f}ms (from a {rows}-row slab)")
     skipped = any("skipped" in s for s in parts)
-    return dict(value=None if skipped else round(total_ms, 1), unit="ms/step", cores=cores, kind="port",
-                sample="one oracle step per distinct Muon shape and one <=4096-row slab per Adam shape, "
+    return dict(value=None if skipped else round(total_ms, 1), unit="ms/step", cores=cores, cpu=cpu_model(), kind="port",
+                sample="one warmed-up oracle step per distinct Muon shape and per <=4096-row slab of each Adam shape, "
                        "summed as count x time (extrapolated): " + ", ".join(parts))
 
 
@@ -234,8 +389,12 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="replay the Muon launches from a HIP graph (use_graph=True): step time only, the "
                          "per-kernel figures need the eager launches")
+    ap.add_argument("--realloc-grads", action="store_true",
+                    help="give every parameter a gradient at a new address each step (as zero_grad("
+                         "set_to_none=True) does), so that re-binding the descriptor tables is timed")
+    ap.add_argument("--no-gates", action="store_true", help="skip the correctness gates (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the secondary GPT-2 measurement")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations (GPT-2, ns32, conv)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run one plain 1 GiB device-to-device copy kernel (a known-size reference "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -245,6 +404,7 @@ def main():
                  "by matrix across ranks, which is not part of this library). Run with --gpus 1.")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X GPU")
+    gates = None if args.no_gates else correctness_gates(args.workload)
     if args.workload == "ns32":
         steps = args.steps if args.steps is not None else 5
         warmup = args.warmup if args.warmup is not None else 1
@@ -256,14 +416,11 @@ def main():
             "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "ns32: zeropower_via_newtonschulz5 on 32 x 4096 x 4096 bf16 ~N(0,1), 5 iterations",
                        "rounding": "reference"},
-            "roofline": {"bound": "mfma", "kernel": "ns_gemm_kernel (syrk + poly + update launches)",
-                         "achieved": round(gemm_work / gemm_ms / 1e9, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(gemm_work / gemm_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                         "launches": gemm_n, "avg_launch_ms": round(gemm_ms / gemm_n, 4),
-                         "flops_per_launch": gemm_work / gemm_n},
+            "gates": gates,
+            "roofline": roofline_object("ns32", gemm_work, gemm_ms, gemm_n),
             "ns": {"tflops_sym_whole_call": round(res["f_sym"] / res["ms_per_step"] / 1e9, 1),
                    "tflops_dense_equiv_whole_call": round(res["f_dense"] / res["ms_per_step"] / 1e9, 1)},
-            "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kernels.items()},
+            "kernels": rounded(kernels),
         }))
         return
     _, _, _, dsteps, dwarm = workload_shapes(args.workload)
@@ -277,16 +434,19 @@ def main():
         torch.cuda.synchronize()
         del a, b
     res = run_optimizer_workload(args.workload, steps, warmup, seed=1234 + 4, ns_variant=args.ns_variant,
-                                 use_graph=args.graph)
+                                 use_graph=args.graph, realloc_grads=args.realloc_grads)
+    grads = "new address every step" if args.realloc_grads else "resident, same addresses every step"
     if args.graph:
         print(json.dumps({"metric": f"muon_step_ms_{args.workload}", "value": round(res["ms_per_step"], 3),
                           "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warmup,
                           "ms_per_step": round(res["ms_per_step"], 3), "higher_is_better": False,
-                          "config": {"workload": args.workload, "ns_variant": args.ns_variant, "launch": "hip graph replay"}}))
+                          "config": {"workload": args.workload, "ns_variant": args.ns_variant, "launch": "hip graph replay",
+                                     "gradients": grads}}))
         return
     kernels, gemm_work, gemm_ms, gemm_n = summarize_kernels(res["per_label"])
     ew_bytes = sum(w for l, (w, ms, n) in res["per_label"].items() if not l.startswith("ns_gemm"))
     ew_ms = sum(ms for l, (w, ms, n) in res["per_label"].items() if not l.startswith("ns_gemm"))
+    alg_bytes = (res["muon_elements"] * 24 + res["adam_elements"] * 28) * steps
     line = {
         "metric": f"muon_step_ms_{args.workload}",
         "value": round(res["ms_per_step"], 3),
@@ -304,19 +464,9 @@ def main():
                                f"{res['muon_elements']} Muon + {res['adam_elements']} Adam elements, "
                                "lr .02 wd .01 momentum .95 nesterov ns_steps 5; Adam lr 3e-4 betas (.9,.95)",
                    "rounding": "reference" if args.ns_variant == "ns5" else "one rounding per stored matrix",
-                   "ns_variant": args.ns_variant},
-        "roofline": {
-            "bound": "mfma",
-            "kernel": "ns_gemm_kernel (syrk + poly + update launches)",
-            "achieved": round(gemm_work / gemm_ms / 1e9, 1),
-            "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(gemm_work / gemm_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
-            "launches": gemm_n,
-            "avg_launch_ms": round(gemm_ms / gemm_n, 4),
-            "flops_per_launch": gemm_work / gemm_n,
-        },
+                   "ns_variant": args.ns_variant, "gradients": grads},
+        "gates": gates,
+        "roofline": roofline_object(args.workload, gemm_work, gemm_ms, gemm_n),
         "ns": {
             "ns_ms_per_step": round(gemm_ms / steps, 3),
             "tflops_sym": round(res["f_sym"] * steps / gemm_ms / 1e9, 1),
@@ -325,17 +475,15 @@ def main():
         "elementwise": {
             "ms_per_step": round(ew_ms / steps, 3),
             "launched_gbs": round(ew_bytes / ew_ms / 1e6, 1),
-            "algorithmic_gbs": round((res["muon_elements"] * 24 + res["adam_elements"] * 28) * steps / ew_ms / 1e6, 1),
-            "frac_of_hbm_peak_algorithmic": round((res["muon_elements"] * 24 + res["adam_elements"] * 28) * steps / ew_ms / 1e6 / PEAK_HBM_GBS, 4),
+            "algorithmic_gbs": round(alg_bytes / ew_ms / 1e6, 1),
+            "frac_of_hbm_peak_algorithmic": round(alg_bytes / ew_ms / 1e6 / PEAK_HBM_GBS, 4),
         },
-        "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in kernels.items()},
+        "kernels": rounded(kernels),
     }
     if not args.no_extra and args.workload == "llama3-8b":
-        g = run_optimizer_workload("gpt2-124m", 10, 3, seed=1234 + 2)
-        _, gw, gms, _ = summarize_kernels(g["per_label"])
-        gg = run_optimizer_workload("gpt2-124m", 10, 3, seed=1234 + 2, use_graph=True)
-        line["gpt2_124m"] = {"ms_per_step": round(g["ms_per_step"], 3), "ns_tflops_sym": round(gw / gms / 1e9, 1),
-                             "ms_per_step_graph_replay": round(gg["ms_per_step"], 3)}
+        line["gpt2_124m"] = secondary("gpt2-124m", not args.no_gates)
+        line["ns32"] = secondary("ns32", not args.no_gates)
+        line["conv"] = secondary("conv", not args.no_gates)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.workload)
         if line["cpu_baseline"]["value"]:

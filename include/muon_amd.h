@@ -139,9 +139,9 @@ typedef struct MuonAolDesc {
 
 int         muon_amd_abi_version(void);
 const char* muon_amd_last_error(void);
-/* One-time set-up on the current device (raises the dynamic LDS limit of the GEMM kernels).
- * Optional -- the first GEMM launch does it too -- but required before recording launches
- * into a HIP graph, because it is not a stream operation.                                   */
+/* One-time set-up on the current device: checks that it is a gfx950 (MUON_AMD_EDEVICE if not),
+ * and raises the dynamic LDS limit of the GEMM kernels.  Optional -- the first GEMM launch on a device does it too -- but required before
+ * recording launches into a HIP graph, because it is not a stream operation.                */
 int         muon_amd_init(void);
 
 /* sizeof() of the structs above, so that a binding can check its own layout. */

@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmuon_amd.so")
+# MUON_AMD_LIBRARY: path of another build of the library (for comparing builds side by side)
+LIB_PATH = os.environ.get("MUON_AMD_LIBRARY") or os.path.join(_HERE, "libmuon_amd.so")
 
 ABI_VERSION = 1
 ROUND_REFERENCE = 1

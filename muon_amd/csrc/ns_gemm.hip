@@ -29,6 +29,9 @@
 
 #include "common.h"
 
+#include <string.h>
+
+#include <mutex>
 #include <vector>
 
 namespace muon_amd {
@@ -288,6 +291,10 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 // multiplied the next one and a half are in flight or landed, the load pipe always has queued
 // requests, and every request is a full 128-byte line.  NHALF = 5 fills the 160 KB LDS for the
 // 256 x 256 tile.
+#ifndef NS_SPLIT_TICKET_ORDER
+#define NS_SPLIT_TICKET_ORDER __ATOMIC_RELEASE
+#endif
+
 template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_, bool SPLIT_K_>
 struct GemmCfg {
     static constexpr bool SPLIT_K = SPLIT_K_;     // jobs may share a tile's reduction
@@ -462,9 +469,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     //      jobs.  Each job parks its fp32 accumulators in its own slot; the job that arrives last
     //      adds the slots in slot order (so the sum does not depend on which job that is) and
     //      writes the tile.  Nobody waits for anybody: the other jobs just exit.
-    //      The slots are written with device-scope stores, which go through to memory past the
-    //      XCD-private L2 (a release fence would write the whole L2 back instead); only the one
-    //      job per tile that adds them up pays for an acquire fence before its plain loads. ------
+    //      Hand-over: the slots are written with device-scope stores, which go through to memory
+    //      past the XCD-private L2; after the workgroup barrier one thread takes the ticket with
+    //      release order at device scope, so every slot store of the workgroup happens before
+    //      the ticket is visible.  Only the one job per tile that adds the slots up pays for an
+    //      acquire fence (which drops what its XCD's L2 holds of them) before its plain loads. ----
     if constexpr (Cfg::SPLIT_K) {
         const int split_count = job.split >> 16;
         if (split_count > 1) {
@@ -479,11 +488,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
                     for (int i = 0; i < 16; ++i)
                         __hip_atomic_store(&mine[lane_off + ((a * TN + b) * 16 + i) * 64], acc[a][b][i],
                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_s_waitcnt(0);                     // my slot has reached memory ...
+            __builtin_amdgcn_s_waitcnt(0);                     // this wave's slot stores are acknowledged ...
             __syncthreads();
             int* const ticket = reinterpret_cast<int*>(lds);
-            if (tid == 0)                                      // ... before I am counted
-                *ticket = __hip_atomic_fetch_add(&split_counters[job.part_base], 1, __ATOMIC_RELAXED,
+            if (tid == 0)                                      // ... and the whole slot is out before I am counted
+                *ticket = __hip_atomic_fetch_add(&split_counters[job.part_base], 1, NS_SPLIT_TICKET_ORDER,
                                                  __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             const bool last = *ticket == split_count - 1;
@@ -546,22 +555,57 @@ static const TileClass kTileClasses[kNumTileClasses] = {
     {Cfg1::BM, Cfg1::BN, Cfg1::NT, Cfg1::LDS_BYTES, Cfg1::SPLIT_K},
 };
 
-// The kernels use more dynamic LDS than the default limit: raised once per process and device
-// function (not a stream operation, so it must not wait for the first launch, which may be one
-// that a caller records into a HIP graph).
+// ---------------------------------------------------------------------------------------------
+// Per-device set-up, done once per device with that device current: the device must be a gfx950,
+// the kernels use more dynamic LDS than the default limit (raising it is not a stream operation,
+// so it must not wait for the first launch, which may be one that a caller records into a HIP
+// graph).
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+    bool ready = false;
+};
+static DeviceState g_devices[kMaxDevices];
+static std::mutex g_devices_mutex;
+
 template <typename Cfg>
 static int raise_lds_limit() {
-    static bool attr_set = false;
-    if (!attr_set) {
-        auto kern = ns_gemm_kernel<Cfg>;
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
-            set_error("ns_gemm: cannot raise dynamic LDS to %zu bytes", Cfg::LDS_BYTES);
-            return MUON_AMD_ELAUNCH;
-        }
-        attr_set = true;
+    auto kern = ns_gemm_kernel<Cfg>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("ns_gemm: cannot raise dynamic LDS to %zu bytes", Cfg::LDS_BYTES);
+        return MUON_AMD_ELAUNCH;
     }
+    return MUON_AMD_OK;
+}
+
+static int device_setup(const DeviceState** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        set_error("no usable HIP device is current (device index %d)", dev);
+        return MUON_AMD_EDEVICE;
+    }
+    std::lock_guard<std::mutex> lock(g_devices_mutex);
+    DeviceState& st = g_devices[dev];
+    if (!st.ready) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("cannot query device %d", dev);
+            return MUON_AMD_EDEVICE;
+        }
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+            set_error("device %d is %s: this library holds gfx950 (MI355X) code only", dev, prop.gcnArchName);
+            return MUON_AMD_EDEVICE;
+        }
+        int rc = raise_lds_limit<Cfg0>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1>();
+        if (rc != MUON_AMD_OK) return rc;
+        st.ready = true;
+    }
+    *out = &st;
     return MUON_AMD_OK;
 }
 
@@ -569,11 +613,17 @@ template <typename Cfg>
 static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
                        float beta, float gamma, int flags, float* split_partials,
                        int32_t* split_counters, hipStream_t s) {
-    const int rc = raise_lds_limit<Cfg>();
-    if (rc != MUON_AMD_OK) return rc;
     hipLaunchKernelGGL(ns_gemm_kernel<Cfg>, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
                        alpha, beta, gamma, flags, split_partials, split_counters);
     return check_launch("ns_gemm");
+}
+
+static int launch_gemm_class(int tile_class, const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs,
+                             float alpha, float beta, float gamma, int flags, float* split_partials,
+                             int32_t* split_counters, hipStream_t s) {
+    if (tile_class == 0)
+        return launch_gemm<Cfg0>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
+    return launch_gemm<Cfg1>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
 }
 
 }  // namespace muon_amd
@@ -583,8 +633,8 @@ using namespace muon_amd;
 extern "C" {
 
 int muon_amd_init(void) {
-    const int rc = raise_lds_limit<Cfg0>();
-    return rc != MUON_AMD_OK ? rc : raise_lds_limit<Cfg1>();
+    const DeviceState* st = nullptr;
+    return device_setup(&st);
 }
 
 int muon_amd_gemm_tile_rows(int tile_class) {
@@ -669,13 +719,11 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
                  "ns_gemm: split partials and counters go together");
     MUON_REQUIRE(njobs > 0, "ns_gemm: njobs=%d", njobs);
     MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "ns_gemm: unknown tile class %d", tile_class);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (tile_class == 0)
-        return launch_gemm<Cfg0>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, split_partials_dev,
-                                 split_counters_dev, s);
-    return launch_gemm<Cfg1>(descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags, split_partials_dev,
-                             split_counters_dev, s);
+    const DeviceState* st = nullptr;
+    const int rc = device_setup(&st);
+    if (rc != MUON_AMD_OK) return rc;
+    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
+                             split_partials_dev, split_counters_dev, static_cast<hipStream_t>(stream));
 }
-
 
 }  // extern "C"

@@ -143,6 +143,11 @@ class _ChunkRuntime:
                         for lay, sz, (has_m, _, _) in zip(c.layouts, store, self.present))
         apply_bytes = sum(lay.numel * (2 + (2 * sz if has_p else 0) + (2 if has_o else 0))
                           for lay, sz, (_, has_p, has_o) in zip(c.layouts, store, self.present))
+        if c.split_slots:
+            # every launch leaves the counters of the split groups zero; clearing them here as well
+            # (a fill kernel, recordable into a graph) keeps a launch that died half way from
+            # poisoning every later step
+            self.split_counters.zero_()
         _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
             int(mutate_grad), sc_mom, s), "momentum"))

@@ -29,17 +29,31 @@ class _MuonBase(torch.optim.Optimizer):
         if ns_variant not in ("ns5", "aol4"):
             raise ValueError(f"ns_variant must be 'ns5' or 'aol4', got {ns_variant!r}")
         self._ns_variant = ns_variant
+        self._ns_rounding = ns_rounding
         self._reference_rounding = _rounding_flag(ns_rounding)
         self._mutate_grad = bool(mutate_grad)
         self._workspace_bytes = workspace_bytes
         self._muon_engines = {}
         self._adam_engines = {}
 
+    _RUNTIME_OPTIONS = ("_ns_rounding", "_mutate_grad", "_workspace_bytes", "_ns_variant", "_use_graph")
+
+    def __getstate__(self):
+        # torch's Optimizer pickles defaults/state/param_groups only; the keyword-only options of
+        # this build select the algorithm (ns_variant, ns_rounding), so a copy must carry them.
+        # Engines (device workspaces, raw addresses, recorded graphs) are rebuilt on the next step.
+        state = super().__getstate__()
+        state["muon_amd_options"] = {k: getattr(self, k) for k in self._RUNTIME_OPTIONS}
+        return state
+
     def __setstate__(self, state):
-        # torch pickles only defaults/state/param_groups; engines (device workspaces and raw
-        # addresses) are rebuilt on the next step.
+        state = dict(state)
+        opts = state.pop("muon_amd_options", None)
         super().__setstate__(state)
-        if not hasattr(self, "_muon_engines"):
+        if opts is not None:
+            self._init_runtime(opts["_ns_rounding"], opts["_mutate_grad"], opts["_workspace_bytes"],
+                               opts["_ns_variant"], opts["_use_graph"])
+        elif not hasattr(self, "_muon_engines"):
             self._init_runtime("reference", False, None)
 
     @staticmethod

@@ -1,0 +1,157 @@
+"""GPU parity of the paths the benchmark runs at the benchmark's own sizes: several chunks sharing
+one workspace (the Llama-3-8B step runs as 4 chunks at the default cap), the full GPT-2-small
+parameter list over 10 steps, 32 x 4096 x 4096 batched Newton-Schulz, and an auxiliary-Adam tensor
+of the Llama-3-8B embedding's size, each against the CPU oracle (or, at sizes the oracle cannot
+reach, through batched == single and slabs of the big tensor)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import muon_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_BF16 = 2e-2
+TOL_PARAM = 1e-3
+TOL_ADAM = 1e-5
+
+
+@pytest.fixture(scope="module")
+def M():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need an MI355X; torch.cuda.is_available() is False")
+    import muon_amd
+    from muon_amd import _lib
+    _lib.load()
+    return muon_amd
+
+
+def _pair(shapes, std, seed):
+    torch.manual_seed(seed)
+    cpu = [torch.nn.Parameter(torch.randn(*s) * std) for s in shapes]
+    gpu = [torch.nn.Parameter(p.detach().clone().cuda()) for p in cpu]
+    return cpu, gpu
+
+
+def _grads(cpu, gpus, std):
+    for i, pc in enumerate(cpu):
+        g = torch.randn_like(pc) * std
+        pc.grad = g.clone()
+        for gpu in gpus:
+            gpu[i].grad = g.clone().cuda()
+
+
+def test_many_chunks_of_both_tile_classes_match_the_oracle_and_the_one_chunk_run(M):
+    """A workspace cap small enough that both tile classes run as several chunks back to back, each
+    reusing the workspace of the one before (the momentum kernel's un-normalised update aliases a
+    transposed-iterate buffer of the previous chunk; split reductions have per-chunk counters):
+    against the oracle, and bit for bit against the same step with everything in one chunk per
+    class.  The sorting class `Muon` runs the steps (muon.py:18-70 at world size 1)."""
+    shapes = [(1024, 2048), (2048, 1024), (768, 768), (256, 576), (128, 8192), (64, 24, 3, 3), (512, 2304),
+              (1280, 1024)]
+    cpu, few = _pair(shapes, 0.02, 1400)
+    many = [torch.nn.Parameter(p.detach().clone()) for p in few]
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    o_few = M.Muon(few, lr=0.02, weight_decay=0.01, momentum=0.95)
+    o_many = M.Muon(many, lr=0.02, weight_decay=0.01, momentum=0.95, workspace_bytes=8 << 20)
+    for step in range(2):
+        _grads(cpu, [few, many], 1e-3)
+        oc.step()
+        o_few.step()
+        o_many.step()
+        for pc, pf, pm in zip(cpu, few, many):
+            assert torch.equal(pf.detach(), pm.detach()), (tuple(pc.shape), step)
+            tol = TOL_PARAM if pc.ndim == 2 else 3e-3        # tiny conv filter: bf16 noise of the update weighs more
+            assert O.rel_fro(pm.detach().cpu(), pc.detach()) <= tol, (tuple(pc.shape), step)
+            np.testing.assert_allclose(o_many.state[pm]["momentum_buffer"].cpu().numpy(),
+                                       oc.state[pc]["momentum_buffer"].numpy(), rtol=1e-6, atol=1e-12)
+    eng_many = next(iter(o_many._muon_engines.values()))
+    eng_few = next(iter(o_few._muon_engines.values()))
+    classes = [rt.chunk.tile_class for rt in eng_many.runtimes]
+    assert classes.count(1) >= 2 and classes.count(0) >= 3, classes
+    assert len(eng_few.runtimes) == 2
+    # the sorting class ordered the group by size, descending (muon.py:42)
+    sizes = [tuple(p.shape) for p in o_many.param_groups[0]["params"]]
+    assert sizes == sorted(sizes, reverse=True)
+
+
+def test_gpt2_small_full_parameter_list_ten_steps(M):
+    """Benchmark configuration 2 at its full list: 12 layers x {768x2304, 768x768, 768x3072, 3072x768}
+    on Muon; wte 50257x768, wpe 1024x768 and 25 vectors of 768 on Adam; gradients ~N(0, 1e-3);
+    10 consecutive steps, every parameter compared with the oracle after the 1st, 5th and 10th."""
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    muon_shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    adam_shapes = [(50257, 768), (1024, 768)] + [(768,)] * 25
+    cpu_m, gpu_m = _pair(muon_shapes, 0.02, 1236)
+    cpu_a, gpu_a = _pair(adam_shapes, 0.02, 1237)
+    mk = lambda cls, pm, pa: cls([dict(params=pm, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01),
+                                  dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)])
+    oc, og = mk(O.OracleSingleDeviceMuonWithAuxAdam, cpu_m, cpu_a), mk(M.SingleDeviceMuonWithAuxAdam, gpu_m, gpu_a)
+    for step in range(10):
+        _grads(cpu_m + cpu_a, [gpu_m + gpu_a], 1e-3)
+        oc.step()
+        og.step()
+        if step in (0, 4, 9):
+            worst = max(O.rel_fro(pg.detach().cpu(), pc.detach()) for pc, pg in zip(cpu_m, gpu_m))
+            print(f"step {step + 1}: worst Muon parameter error {worst:.2e}")
+            # The 1e-3 bound is stated for one full step.  Each step's update carries its own bf16
+            # Newton-Schulz noise (within 2e-2 of the update, independent from step to step), so
+            # after k steps the distance has grown like a random walk: the bound is 1e-3 * sqrt(k).
+            assert worst <= TOL_PARAM * (step + 1) ** 0.5, step
+            for pc, pg in zip(cpu_a, gpu_a):
+                np.testing.assert_allclose(pg.detach().cpu().numpy(), pc.detach().numpy(), rtol=TOL_ADAM, atol=1e-8)
+    assert og.state[gpu_a[0]]["step"] == 10
+
+
+def test_batch_of_32_square_matrices_equals_single_runs(M):
+    """Benchmark configuration 3 at its full batch: 32 x 4096 x 4096 bf16 ~N(0,1).  The batched call
+    returns, for a sample of indices, the bits of the one-matrix call, and one matrix is compared
+    with the oracle's bf16 restatement."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1237)
+    G = torch.randn(32, 4096, 4096, device="cuda", generator=gen).bfloat16()
+    out = M.zeropower_via_newtonschulz5(G)
+    assert out.shape == G.shape and out.dtype == torch.bfloat16
+    for b in (0, 13, 31):
+        assert torch.equal(M.zeropower_via_newtonschulz5(G[b]), out[b]), b
+    fro = out.float().flatten(1).norm(dim=1)
+    assert torch.isfinite(fro).all() and float(fro.min()) > 0.5 * 64 and float(fro.max()) < 1.2 * 64   # singular values in (0.5, 1.2)
+    torch.set_num_threads(min(16, os.cpu_count() or 1))
+    assert O.rel_fro(out[7].float().cpu(), O.ns5_bf16(G[7].cpu()).float()) <= TOL_BF16
+    M.clear_engine_cache()
+
+
+def test_embedding_sized_adam_tensor_slabs(M):
+    """A 128256 x 4096 auxiliary-Adam tensor (Llama-3-8B embed / lm_head: 525 M elements, byte
+    offsets beyond 2^31): two steps on the GPU, the first, a middle and the last 4096 rows against
+    the oracle run on those rows (the update is elementwise), plus the 4096-vector class."""
+    rows, cols, slab = 128256, 4096, 4096
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1410)
+    p = torch.nn.Parameter(torch.randn(rows, cols, device="cuda", generator=gen) * 0.02)
+    v = torch.nn.Parameter(torch.ones(cols, device="cuda"))
+    starts = [0, (rows // 2 // 8) * 8 + 3, rows - slab]            # one slab at an odd row offset
+    cpu = [torch.nn.Parameter(p.detach()[s:s + slab].cpu().clone()) for s in starts]
+    cpu_v = torch.nn.Parameter(v.detach().cpu().clone())
+    kw = dict(use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)
+    og = M.SingleDeviceMuonWithAuxAdam([dict(params=[p, v], **kw)])
+    oc = O.OracleSingleDeviceMuonWithAuxAdam([dict(params=cpu + [cpu_v], **kw)])
+    for step in range(2):
+        g = torch.randn(rows, cols, device="cuda", generator=gen) * 1e-4
+        gv = torch.randn(cols, device="cuda", generator=gen) * 1e-4
+        p.grad, v.grad = g, gv
+        for s, pc in zip(starts, cpu):
+            pc.grad = g[s:s + slab].cpu()
+        cpu_v.grad = gv.cpu()
+        og.step()
+        oc.step()
+        torch.cuda.synchronize()
+        for s, pc in zip(starts, cpu):
+            np.testing.assert_allclose(p.detach()[s:s + slab].cpu().numpy(), pc.detach().numpy(), rtol=TOL_ADAM, atol=1e-9)
+            for key in ("exp_avg", "exp_avg_sq"):
+                np.testing.assert_allclose(og.state[p][key][s:s + slab].cpu().numpy(), oc.state[pc][key].numpy(),
+                                           rtol=TOL_ADAM, atol=1e-16)
+        np.testing.assert_allclose(v.detach().cpu().numpy(), cpu_v.detach().numpy(), rtol=TOL_ADAM, atol=1e-9)
+        del g

@@ -219,6 +219,25 @@ def test_constructor_contract_matches_the_reference():
         muon_amd.SingleDeviceMuon([a], ns_rounding="nearest")
 
 
+def test_copies_and_pickles_keep_the_algorithm_options():
+    """torch pickles only defaults/state/param_groups; the keyword-only options that select the
+    algorithm must survive copy.deepcopy and pickle, or a copied optimizer silently runs another
+    iteration."""
+    import copy
+    import pickle
+    a = torch.nn.Parameter(torch.zeros(4, 8))
+    opt = muon_amd.SingleDeviceMuon([a], ns_variant="aol4", ns_rounding="fused", mutate_grad=True,
+                                    use_graph=True, workspace_bytes=1 << 20)
+    for dup in (copy.deepcopy(opt), pickle.loads(pickle.dumps(opt))):
+        assert dup._ns_variant == "aol4" and dup._reference_rounding is False
+        assert dup._mutate_grad is True and dup._use_graph is True and dup._workspace_bytes == 1 << 20
+        assert dup._muon_engines == {} and dup.param_groups[0]["lr"] == 0.02
+    aux = muon_amd.MuonWithAuxAdam([dict(params=[a], use_muon=True)], ns_variant="aol4")
+    assert copy.deepcopy(aux)._ns_variant == "aol4"
+    plain = copy.deepcopy(muon_amd.SingleDeviceMuon([a]))
+    assert plain._ns_variant == "ns5" and plain._reference_rounding is True and plain._use_graph is False
+
+
 def test_no_cpu_fallback():
     a = torch.nn.Parameter(torch.zeros(4, 8))
     a.grad = torch.ones(4, 8)
