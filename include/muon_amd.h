@@ -140,7 +140,8 @@ typedef struct MuonAolDesc {
 int         muon_amd_abi_version(void);
 const char* muon_amd_last_error(void);
 /* One-time set-up on the current device: checks that it is a gfx950 (MUON_AMD_EDEVICE if not),
- * and raises the dynamic LDS limit of the GEMM kernels.  Optional -- the first GEMM launch on a device does it too -- but required before
+ * raises the dynamic LDS limit of the GEMM kernels and looks up the device's static scratch
+ * array.  Optional -- the first GEMM launch on a device does it too -- but required before
  * recording launches into a HIP graph, because it is not a stream operation.                */
 int         muon_amd_init(void);
 
@@ -171,6 +172,23 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs_host, int ndesc,
 int muon_amd_validate_mats(const MuonMatDesc* descs_host, int nmat,
                            const int32_t* block_prefix_host, const int32_t* tile_prefix_host,
                            int tile_edge);
+
+/* The same launch for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The fp32 slots and counters of split reductions live in a static device array inside the
+ * library (MUON_AMD_NOALLOC_MAX_SPLIT_SLOTS slots of 128 x 128 floats plus one counter each,
+ * 16 MiB + 1 KiB per GPU, held until the process ends) instead of caller-owned memory; the call
+ * clears the counters it uses with a small fill kernel on `stream`, then enqueues the same
+ * kernel as muon_amd_ns_gemm.  split_slots = number of slots the job list addresses (0 when no
+ * job is split; the value given to muon_amd_validate_gemm); more than the maximum is refused
+ * with MUON_AMD_EINVAL.  It allocates and frees nothing.  All calls on one GPU share that GPU's
+ * array: two calls with split jobs whose kernels overlap on one GPU (different streams, or
+ * different threads) race; calls on one stream are ordered and safe.                          */
+#define MUON_AMD_NOALLOC_MAX_SPLIT_SLOTS 256
+int muon_amd_noalloc_max_split_slots(void);
+int muon_amd_ns_gemm_noalloc(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
+                             int tile_class, float alpha, float beta, float gamma, int flags,
+                             int split_slots, void* stream);
 
 /* ---- Muon elementwise stages ------------------------------------------------------------ */
 

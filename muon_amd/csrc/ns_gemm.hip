@@ -559,11 +559,22 @@ static const TileClass kTileClasses[kNumTileClasses] = {
 // Per-device set-up, done once per device with that device current: the device must be a gfx950,
 // the kernels use more dynamic LDS than the default limit (raising it is not a stream operation,
 // so it must not wait for the first launch, which may be one that a caller records into a HIP
-// graph).
+// graph), and the address of this device's copy of the static scratch array is looked up.
 // ---------------------------------------------------------------------------------------------
+// Split-reduction scratch for callers that cannot allocate (muon_amd_ns_gemm_noalloc): the fp32
+// slots of the 128 x 128 tile class followed by one int32 counter per slot.  Every GPU the
+// library runs on holds its own copy until the process ends.  In host code the name `scratch`
+// is only a handle for hipGetSymbolAddress; kernels are given the looked-up address.
+constexpr int kStaticSplitSlots = MUON_AMD_NOALLOC_MAX_SPLIT_SLOTS;
+constexpr size_t kStaticSlotBytes = static_cast<size_t>(Cfg0::BM) * Cfg0::BN * sizeof(float);
+constexpr size_t kStaticCounterOffset = kStaticSplitSlots * kStaticSlotBytes;
+constexpr size_t kStaticScratchBytes = kStaticCounterOffset + kStaticSplitSlots * sizeof(int32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 constexpr int kMaxDevices = 64;
 struct DeviceState {
     bool ready = false;
+    unsigned char* scratch_ptr = nullptr;     // device address of `scratch` on this device
 };
 static DeviceState g_devices[kMaxDevices];
 static std::mutex g_devices_mutex;
@@ -603,6 +614,13 @@ static int device_setup(const DeviceState** out) {
         int rc = raise_lds_limit<Cfg0>();
         if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1>();
         if (rc != MUON_AMD_OK) return rc;
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            set_error("cannot look up the static scratch array on device %d", dev);
+            return MUON_AMD_ELAUNCH;
+        }
+        st.scratch_ptr = static_cast<unsigned char*>(ptr);
         st.ready = true;
     }
     *out = &st;
@@ -624,6 +642,11 @@ static int launch_gemm_class(int tile_class, const MuonGemmDesc* descs, const Mu
     if (tile_class == 0)
         return launch_gemm<Cfg0>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
     return launch_gemm<Cfg1>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
+}
+
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
 }
 
 }  // namespace muon_amd
@@ -724,6 +747,37 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
     if (rc != MUON_AMD_OK) return rc;
     return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
                              split_partials_dev, split_counters_dev, static_cast<hipStream_t>(stream));
+}
+
+int muon_amd_noalloc_max_split_slots(void) { return kStaticSplitSlots; }
+
+int muon_amd_ns_gemm_noalloc(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
+                             int tile_class, float alpha, float beta, float gamma, int flags,
+                             int split_slots, void* stream) {
+    MUON_REQUIRE(descs_dev && jobs_dev, "ns_gemm_noalloc: null table");
+    MUON_REQUIRE(njobs > 0, "ns_gemm_noalloc: njobs=%d", njobs);
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "ns_gemm_noalloc: unknown tile class %d", tile_class);
+    MUON_REQUIRE(split_slots >= 0, "ns_gemm_noalloc: split_slots=%d", split_slots);
+    MUON_REQUIRE(split_slots <= kStaticSplitSlots,
+                 "ns_gemm_noalloc: the job list uses %d split slots, the static scratch holds %d "
+                 "(use muon_amd_ns_gemm with a caller-owned workspace)", split_slots, kStaticSplitSlots);
+    MUON_REQUIRE(split_slots == 0 || kTileClasses[tile_class].split_k,
+                 "ns_gemm_noalloc: tile class %d does not split reductions", tile_class);
+    const DeviceState* st = nullptr;
+    const int rc = device_setup(&st);
+    if (rc != MUON_AMD_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float* const partials = reinterpret_cast<float*>(st->scratch_ptr);
+    int32_t* const counters = reinterpret_cast<int32_t*>(st->scratch_ptr + kStaticCounterOffset);
+    if (split_slots > 0) {
+        // The array keeps whatever the last call left: the counters must start at zero.  A small
+        // fill kernel rather than a memset node, so that the call can be recorded into a HIP graph.
+        hipLaunchKernelGGL(zero_i32_kernel, dim3((split_slots + 255) / 256), dim3(256), 0, s, counters, split_slots);
+        const int zrc = check_launch("ns_gemm_noalloc: clear counters");
+        if (zrc != MUON_AMD_OK) return zrc;
+    }
+    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
+                             split_slots > 0 ? partials : nullptr, split_slots > 0 ? counters : nullptr, s);
 }
 
 }  // extern "C"
