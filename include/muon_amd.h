@@ -173,6 +173,23 @@ int muon_amd_validate_mats(const MuonMatDesc* descs_host, int nmat,
                            const int32_t* block_prefix_host, const int32_t* tile_prefix_host,
                            int tile_edge);
 
+/* The last update product of the iteration with the parameter step fused into its epilogue
+ * (muon.py:287 followed by muon.py:14, 98-99, 15): for every matrix k of the launch, with
+ * o = bf16(alpha*acc + beta*D) as above,
+ *     update = bf16(o * mats[k].scale);
+ *     mats[k].param <- mats[k].param * wd_factor - lr * update     (if param)
+ *     mats[k].out   <- update                                      (if out)
+ * in the storage type mats[k].src_dtype, at the unpadded extent mats[k].rows x mats[k].cols.
+ * X is the parameter itself for a wide matrix (rows <= cols) and its transpose for a tall one; the
+ * C / CT / C2 / C2T pointers of the descriptors are ignored (nothing else is written), jobs are
+ * never split.  mats_dev is the table of the elementwise launches; it is indexed by
+ * MuonTileJob.desc.  scalars_dev: NULL or device memory holding {lr, wd_factor} (see
+ * muon_amd_momentum).                                                                        */
+int muon_amd_ns_gemm_apply(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
+                           int tile_class, float alpha, float beta, int flags,
+                           const MuonMatDesc* mats_dev, float lr, float wd_factor,
+                           const float* scalars_dev, void* stream);
+
 /* The same launch for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * The fp32 slots and counters of split reductions live in a static device array inside the

@@ -74,6 +74,7 @@ SIGNATURES = {
     "muon_amd_norm_finalize": (_c_int, [_vp, _c_int, _c_float, _c_int, _vp]),
     "muon_amd_normalize": (_c_int, [_vp, _vp, _c_int, _c_int, _vp]),
     "muon_amd_ns_gemm": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _vp, _vp, _vp]),
+    "muon_amd_ns_gemm_apply": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_int, _vp, _c_float, _c_float, _vp, _vp]),
     "muon_amd_noalloc_max_split_slots": (_c_int, []),
     "muon_amd_ns_gemm_noalloc": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int, _vp]),
     "muon_amd_apply": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _c_float, _vp, _vp]),

@@ -118,26 +118,109 @@ __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 v, float gamma) {
     return r;
 }
 
-// Wave-private staging bytes the epilogue needs for a WM x WN wave tile (rows padded by 16 B).
+// Wave-private staging bytes the epilogue needs for a WM x WN wave tile: the whole addend piece
+// (WM rows of 128 bytes) while it is read into registers, then one 32-row strip of results in
+// each orientation (rows padded by 16 bytes).
 constexpr int epilogue_stage_bytes(int WM, int WN) {
-    return (WM * (WN * 2 + 16) > WN * (WM * 2 + 16)) ? WM * (WN * 2 + 16) : WN * (WM * 2 + 16);
+    return (WM * 128 > 32 * (WN * 2 + 16) + WN * (32 * 2 + 16)) ? WM * 128 : 32 * (WN * 2 + 16) + WN * (32 * 2 + 16);
 }
 
-// Per 32 x 32 tile: t1 = alpha*acc -> row-owning layout -> + beta*D (8-byte loads) -> o (bf16)
-// -> staged row-major in LDS -> 16-byte coalesced stores of C (and gamma*o to C2); o moved back
-// to the column-owning layout -> staged -> 16-byte coalesced stores of CT (and C2T).
-template <bool HAS_D, bool STREAM, int WGN, int WM, int WN, int TM, int TN>
+// The parameter step fused into the epilogue of the last update product (muon.py:14, 98-99):
+//     update = bf16(o * scale);  param <- param * wd_factor - lr * update;  out <- update
+// for 8 consecutive elements of parameter row `prow` starting at column `pcol`, o packed as bf16.
+// The arithmetic is apply_kernel's (elementwise.hip), in the storage type of the parameter.
+struct ApplyArgs {
+    const MuonMatDesc* mat;
+    float neg_lr, wd_factor;
+    bool vec_ok;          // 16-byte accesses are possible: cols % 8 == 0 and aligned base pointers
+};
+
+__device__ __forceinline__ void apply_chunk8(const ApplyArgs& ap, int prow, int pcol, u32x4 v) {
+    const MuonMatDesc& m = *ap.mat;
+    if (prow >= m.rows || pcol >= m.cols) return;          // padding rows / columns of the tile grid
+    float us[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        us[2 * k] = round_bf(__uint_as_float(v[k] << 16) * m.scale);
+        us[2 * k + 1] = round_bf(__uint_as_float(v[k] & 0xffff0000u) * m.scale);
+    }
+    const int64_t e = static_cast<int64_t>(prow) * m.cols + pcol;
+    const bool full = ap.vec_ok && pcol + 8 <= m.cols;
+    const int nvalid = m.cols - pcol < 8 ? m.cols - pcol : 8;
+    if (m.param) {
+        if (m.src_dtype == MUON_AMD_SRC_BF16) {
+            uint16_t* const p = static_cast<uint16_t*>(m.param) + e;
+            if (full) {
+                const u32x4 pv = __builtin_nontemporal_load((const __attribute__((address_space(1))) u32x4*)(p));
+                u32x4 r;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float lo = round_bf(fmaf(ap.neg_lr, us[2 * k], round_bf(__uint_as_float(pv[k] << 16) * ap.wd_factor)));
+                    const float hi = round_bf(fmaf(ap.neg_lr, us[2 * k + 1], round_bf(__uint_as_float(pv[k] & 0xffff0000u) * ap.wd_factor)));
+                    r[k] = pack2bf(lo, hi);
+                }
+                __builtin_nontemporal_store(r, (__attribute__((address_space(1))) u32x4*)(p));
+            } else {
+                for (int k = 0; k < nvalid; ++k)
+                    p[k] = f2bf(fmaf(ap.neg_lr, us[k], round_bf(bf2f(p[k]) * ap.wd_factor)));
+            }
+        } else {
+            float* const p = static_cast<float*>(m.param) + e;
+            if (full) {
+                typedef float f32x4g __attribute__((ext_vector_type(4)));
+                f32x4g p0 = __builtin_nontemporal_load((const __attribute__((address_space(1))) f32x4g*)(p));
+                f32x4g p1 = __builtin_nontemporal_load((const __attribute__((address_space(1))) f32x4g*)(p + 4));
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    p0[k] = fmaf(ap.neg_lr, us[k], p0[k] * ap.wd_factor);
+                    p1[k] = fmaf(ap.neg_lr, us[4 + k], p1[k] * ap.wd_factor);
+                }
+                __builtin_nontemporal_store(p0, (__attribute__((address_space(1))) f32x4g*)(p));
+                __builtin_nontemporal_store(p1, (__attribute__((address_space(1))) f32x4g*)(p + 4));
+            } else {
+                for (int k = 0; k < nvalid; ++k) p[k] = fmaf(ap.neg_lr, us[k], p[k] * ap.wd_factor);
+            }
+        }
+    }
+    if (m.out) {
+        uint16_t* const o = m.out + e;
+        if (full) {
+            u32x4 r;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) r[k] = pack2bf(us[2 * k], us[2 * k + 1]);
+            *(__attribute__((address_space(1))) u32x4*)(o) = r;
+        } else {
+            for (int k = 0; k < nvalid; ++k) o[k] = f2bf(us[k]);
+        }
+    }
+}
+
+// Per 32-row strip of the wave's sub-tile, per 32 x 32 tile of it: t1 = alpha*acc -> row-owning
+// layout -> + beta*D -> o (bf16) -> staged row-major in LDS -> 16-byte coalesced stores of C (and
+// gamma*o to C2); o moved back to the column-owning layout -> staged -> 16-byte coalesced stores
+// of CT (and C2T).  With APPLY, the orientation of the parameter goes through the fused parameter
+// step instead of a store, and the other orientation is not produced.
+template <bool HAS_D, bool STREAM, bool APPLY, int WGN, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const MuonGemmDesc& d,
                                                  const MuonTileJob& job, float alpha, float beta,
-                                                 float gamma, bool round_terms, char* stage) {
-    constexpr int DROW = WN * 2 + 16;   // staged row pitch in bytes, direct orientation
-    constexpr int TROW = WM * 2 + 16;   // transposed orientation
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                                                 float gamma, bool round_terms, char* stage,
+                                                 const ApplyArgs& ap) {
+    constexpr int DROW = WN * 2 + 16;   // staged row pitch in bytes, direct orientation (32 rows)
+    constexpr int TROW = 32 * 2 + 16;   // transposed orientation (WN rows of one strip's 32 columns)
+    constexpr int TOFF = 32 * DROW;     // the transposed strip sits behind the direct one
+    // The thread index goes through an opaque move here: everything the epilogue derives from it
+    // is then computed after the main loop instead of being hoisted above it, where it would sit
+    // in registers the loop needs (and be spilled to scratch memory by every wave).
+    int tid_e = threadIdx.x;
+    asm volatile("" : "+v"(tid_e));
+    const int lane = tid_e & 63, wave = __builtin_amdgcn_readfirstlane(tid_e >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int lr = lane & 31, g = lane >> 5;
     const int row0 = job.i0 + wm * WM, col0 = job.j0 + wn * WN;   // origin of this wave's sub-tile
-    const bool do_d = d.C != nullptr;
-    const bool do_t = d.CT != nullptr && !(job.diag && d.CT == d.C);
+    // X is the parameter itself for a wide parameter and its transpose for a tall one
+    const bool apply_t = APPLY && ap.mat->rows > ap.mat->cols;
+    const bool do_d = APPLY ? !apply_t : d.C != nullptr;
+    const bool do_t = APPLY ? apply_t : (d.CT != nullptr && !(job.diag && d.CT == d.C));
 
     bf16x8 id0, id1;
 #pragma unroll
@@ -182,9 +265,9 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
         // below overwrite the area)
     }
 
-    uint32_t ot[TM][TN][8];   // results moved back to accumulator layout, packed bf16 pairs
 #pragma unroll
     for (int a = 0; a < TM; ++a) {
+        uint32_t ot[TN][8];   // this strip's results moved back to accumulator layout, packed bf16 pairs
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
             f32x16 u;
@@ -227,54 +310,65 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
                     u32x2 pk;
                     pk.x = pack2bf(o[4 * q], o[4 * q + 1]);
                     pk.y = pack2bf(o[4 * q + 2], o[4 * q + 3]);
-                    *reinterpret_cast<u32x2*>(stage + (a * 32 + lr) * DROW + (b * 32 + 8 * q + 4 * g) * 2) = pk;
+                    *reinterpret_cast<u32x2*>(stage + lr * DROW + (b * 32 + 8 * q + 4 * g) * 2) = pk;
                 }
             }
             if (do_t) {
                 const f32x16 w = tile_transpose_bf16(o, id0, id1);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) ot[a][b][k] = pack2bf(w[2 * k], w[2 * k + 1]);
+                for (int k = 0; k < 8; ++k) ot[b][k] = pack2bf(w[2 * k], w[2 * k + 1]);
             }
         }
-    }
-
-    if (do_d) {
-        // 16-byte chunks per row, whole rows per wave-wide store (lanes beyond RPI rows idle)
-        constexpr int CPR = WN / 8, RPI = 64 / CPR;
-        const int r = lane / CPR, ch = lane % CPR;
+        if (do_d) {
+            // 16-byte chunks per row, whole rows per wave-wide store
+            constexpr int CPR = WN / 8, RPI = 64 / CPR;
+            const int r = lane / CPR, ch = lane % CPR;
+            if constexpr (APPLY) {
+#pragma unroll 1
+                for (int it = 0; it < 32 / RPI; ++it) {
+                    const int row = it * RPI + r;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
+                    apply_chunk8(ap, row0 + a * 32 + row, col0 + ch * 8, v);
+                }
+            } else {
 #pragma unroll
-        for (int it = 0; it < (WM + RPI - 1) / RPI; ++it) {
-            const int row = it * RPI + r;
-            if (r < RPI && row < WM) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
-                const size_t off = static_cast<size_t>(row0 + row) * d.ldc + col0 + ch * 8;
-                gstore16<STREAM>(d.C + off, v);
-                if (d.C2) gstore16<STREAM>(d.C2 + off, scale_bf16x8(v, gamma));
+                for (int it = 0; it < 32 / RPI; ++it) {
+                    const int row = it * RPI + r;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * DROW + ch * 16);
+                    const size_t off = static_cast<size_t>(row0 + a * 32 + row) * d.ldc + col0 + ch * 8;
+                    gstore16<STREAM>(d.C + off, v);
+                    if (d.C2) gstore16<STREAM>(d.C2 + off, scale_bf16x8(v, gamma));
+                }
             }
         }
-    }
-    if (do_t) {
-#pragma unroll
-        for (int a = 0; a < TM; ++a)
+        if (do_t) {
 #pragma unroll
             for (int b = 0; b < TN; ++b)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     u32x2 pk;
-                    pk.x = ot[a][b][2 * q];
-                    pk.y = ot[a][b][2 * q + 1];
-                    *reinterpret_cast<u32x2*>(stage + (b * 32 + lr) * TROW + (a * 32 + 8 * q + 4 * g) * 2) = pk;
+                    pk.x = ot[b][2 * q];
+                    pk.y = ot[b][2 * q + 1];
+                    *reinterpret_cast<u32x2*>(stage + TOFF + (b * 32 + lr) * TROW + (8 * q + 4 * g) * 2) = pk;
                 }
-        constexpr int CPR = WM / 8, RPI = 64 / CPR;
-        const int r = lane / CPR, ch = lane % CPR;
+            constexpr int CPR = 32 / 8, RPI = 64 / CPR;
+            const int r = lane / CPR, ch = lane % CPR;
+            if constexpr (APPLY) {
+#pragma unroll 1
+                for (int it = 0; it < WN / RPI; ++it) {
+                    const int row = it * RPI + r;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + TOFF + row * TROW + ch * 16);
+                    apply_chunk8(ap, col0 + row, row0 + a * 32 + ch * 8, v);
+                }
+            } else {
 #pragma unroll
-        for (int it = 0; it < (WN + RPI - 1) / RPI; ++it) {
-            const int row = it * RPI + r;
-            if (r < RPI && row < WN) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
-                const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + ch * 8;
-                gstore16<STREAM>(d.CT + off, v);
-                if (d.C2T) gstore16<STREAM>(d.C2T + off, scale_bf16x8(v, gamma));
+                for (int it = 0; it < WN / RPI; ++it) {
+                    const int row = it * RPI + r;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + TOFF + row * TROW + ch * 16);
+                    const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + a * 32 + ch * 8;
+                    gstore16<STREAM>(d.CT + off, v);
+                    if (d.C2T) gstore16<STREAM>(d.C2T + off, scale_bf16x8(v, gamma));
+                }
             }
         }
     }
@@ -314,11 +408,15 @@ struct GemmCfg {
     static_assert(LDS_BYTES <= 163840, "LDS capacity of a gfx950 CU");
 };
 
-template <typename Cfg>
+// APPLY: the launch is the last update product of the iteration and its epilogue takes the
+// parameter step (mats[job.desc] describes the parameter of the job's matrix; `sc`, when given,
+// holds {lr, wd_factor} in device memory and overrides the by-value arguments).
+template <typename Cfg, bool APPLY>
 __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, float alpha,
     float beta, float gamma, int flags, float* __restrict__ split_partials,
-    int32_t* __restrict__ split_counters) {
+    int32_t* __restrict__ split_counters, const MuonMatDesc* __restrict__ mats, float neg_lr,
+    float wd_factor, const float* __restrict__ sc) {
     constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
     constexpr int NHALF = Cfg::NHALF;
@@ -530,8 +628,18 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     }
     char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
     const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
-    if (d.D) ns_epilogue_impl<true, Cfg::STREAM_STORES, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
-    else ns_epilogue_impl<false, Cfg::STREAM_STORES, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage);
+    ApplyArgs ap{nullptr, 0.f, 1.f, false};
+    if constexpr (APPLY) {
+        ap.mat = mats + job.desc;
+        ap.neg_lr = sc ? -sc[0] : neg_lr;
+        ap.wd_factor = sc ? sc[1] : wd_factor;
+        ap.vec_ok = (ap.mat->cols % 8 == 0) && ((reinterpret_cast<uintptr_t>(ap.mat->param) & 15) == 0) &&
+                    ((reinterpret_cast<uintptr_t>(ap.mat->out) & 15) == 0);
+        ns_epilogue_impl<true, Cfg::STREAM_STORES, true, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
+    } else {
+        if (d.D) ns_epilogue_impl<true, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
+        else ns_epilogue_impl<false, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
+    }
 }
 
 // Tile classes: square output tile, waves, workgroups per CU.
@@ -579,9 +687,9 @@ struct DeviceState {
 static DeviceState g_devices[kMaxDevices];
 static std::mutex g_devices_mutex;
 
-template <typename Cfg>
+template <typename Cfg, bool APPLY>
 static int raise_lds_limit() {
-    auto kern = ns_gemm_kernel<Cfg>;
+    auto kern = ns_gemm_kernel<Cfg, APPLY>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
         (void)hipGetLastError();
@@ -611,8 +719,10 @@ static int device_setup(const DeviceState** out) {
             set_error("device %d is %s: this library holds gfx950 (MI355X) code only", dev, prop.gcnArchName);
             return MUON_AMD_EDEVICE;
         }
-        int rc = raise_lds_limit<Cfg0>();
-        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1>();
+        int rc = raise_lds_limit<Cfg0, false>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg0, true>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, false>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, true>();
         if (rc != MUON_AMD_OK) return rc;
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
@@ -627,21 +737,33 @@ static int device_setup(const DeviceState** out) {
     return MUON_AMD_OK;
 }
 
+struct ApplyLaunch {            // the fused parameter step of the last update product, or mats == nullptr
+    const MuonMatDesc* mats;
+    float neg_lr, wd_factor;
+    const float* scalars;
+};
+
 template <typename Cfg>
 static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
                        float beta, float gamma, int flags, float* split_partials,
-                       int32_t* split_counters, hipStream_t s) {
-    hipLaunchKernelGGL(ns_gemm_kernel<Cfg>, dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
-                       alpha, beta, gamma, flags, split_partials, split_counters);
+                       int32_t* split_counters, const ApplyLaunch& ap, hipStream_t s) {
+    if (ap.mats)
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, true>), dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                           alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
+                           ap.wd_factor, ap.scalars);
+    else
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false>), dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                           alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
+                           ap.wd_factor, ap.scalars);
     return check_launch("ns_gemm");
 }
 
 static int launch_gemm_class(int tile_class, const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs,
                              float alpha, float beta, float gamma, int flags, float* split_partials,
-                             int32_t* split_counters, hipStream_t s) {
+                             int32_t* split_counters, const ApplyLaunch& ap, hipStream_t s) {
     if (tile_class == 0)
-        return launch_gemm<Cfg0>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
-    return launch_gemm<Cfg1>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, s);
+        return launch_gemm<Cfg0>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
+    return launch_gemm<Cfg1>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
 }
 
 __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, int n) {
@@ -746,7 +868,22 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
     const int rc = device_setup(&st);
     if (rc != MUON_AMD_OK) return rc;
     return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
-                             split_partials_dev, split_counters_dev, static_cast<hipStream_t>(stream));
+                             split_partials_dev, split_counters_dev, ApplyLaunch{nullptr, 0.f, 1.f, nullptr},
+                             static_cast<hipStream_t>(stream));
+}
+
+int muon_amd_ns_gemm_apply(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev, int njobs,
+                           int tile_class, float alpha, float beta, int flags,
+                           const MuonMatDesc* mats_dev, float lr, float wd_factor,
+                           const float* scalars_dev, void* stream) {
+    MUON_REQUIRE(descs_dev && jobs_dev && mats_dev, "ns_gemm_apply: null table");
+    MUON_REQUIRE(njobs > 0, "ns_gemm_apply: njobs=%d", njobs);
+    MUON_REQUIRE(tile_class >= 0 && tile_class < kNumTileClasses, "ns_gemm_apply: unknown tile class %d", tile_class);
+    const DeviceState* st = nullptr;
+    const int rc = device_setup(&st);
+    if (rc != MUON_AMD_OK) return rc;
+    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, 0.f, flags, nullptr, nullptr,
+                             ApplyLaunch{mats_dev, -lr, wd_factor, scalars_dev}, static_cast<hipStream_t>(stream));
 }
 
 int muon_amd_noalloc_max_split_slots(void) { return kStaticSplitSlots; }
@@ -777,7 +914,8 @@ int muon_amd_ns_gemm_noalloc(const MuonGemmDesc* descs_dev, const MuonTileJob* j
         if (zrc != MUON_AMD_OK) return zrc;
     }
     return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
-                             split_slots > 0 ? partials : nullptr, split_slots > 0 ? counters : nullptr, s);
+                             split_slots > 0 ? partials : nullptr, split_slots > 0 ? counters : nullptr,
+                             ApplyLaunch{nullptr, 0.f, 1.f, nullptr}, s);
 }
 
 }  // extern "C"

@@ -9,6 +9,9 @@ import torch
 from . import _lib, plan as _plan
 
 DEFAULT_WORKSPACE_CAP = int(os.environ.get("MUON_AMD_WORKSPACE_BYTES", 16 << 30))
+# Measurement knob: 0 runs the parameter step as a launch of its own after the last update product
+# instead of inside that product's epilogue.
+FOLD_APPLY = os.environ.get("MUON_AMD_FOLD_APPLY", "1") != "0"
 
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
@@ -183,8 +186,16 @@ class _ChunkRuntime:
                     self.aol_ptr, self.aol_seg_prefix_ptr, c.nmat, int(c.aol_seg_prefix[-1]), s),
                     "aol_rescale"))
             gemm("ns_gemm/poly", _plan.PH_POLY, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_POLY])
+            if it == c.steps - 1 and FOLD_APPLY:
+                # the last update product takes the parameter step in its epilogue (muon.py:14, 98-99)
+                al, be, _ = c.phase_scalars(_plan.PH_UPD_LAST, it)
+                _launch("ns_gemm/update_apply", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm_apply(
+                    self.gemm_ptr[_plan.PH_UPD_LAST], self.full_jobs_ptr, len(c.full_jobs), c.tile_class, al, be,
+                    flags, mats, lr, wd_factor, sc_apply, s), "ns_gemm_apply"))
+                return
             ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
             gemm("ns_gemm/update", ph, it, self.full_jobs_ptr, len(c.full_jobs), f_upd)
+        # no iteration (steps == 0), or the fused step switched off: a launch of its own
         _launch("apply", apply_bytes, lambda: _lib.check(lib.muon_amd_apply(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, sc_apply, s), "apply"))
 
