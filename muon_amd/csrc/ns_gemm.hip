@@ -118,13 +118,6 @@ __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 v, float gamma) {
     return r;
 }
 
-// Wave-private staging bytes the epilogue needs for a WM x WN wave tile: the whole addend piece
-// (WM rows of 128 bytes) while it is read into registers, then one 32-row strip of results in
-// each orientation (rows padded by 16 bytes).
-constexpr int epilogue_stage_bytes(int WM, int WN) {
-    return (WM * 128 > 32 * (WN * 2 + 16) + WN * (32 * 2 + 16)) ? WM * 128 : 32 * (WN * 2 + 16) + WN * (32 * 2 + 16);
-}
-
 // The parameter step fused into the epilogue of the last update product (muon.py:14, 98-99):
 //     update = bf16(o * scale);  param <- param * wd_factor - lr * update;  out <- update
 // for 8 consecutive elements of parameter row `prow` starting at column `pcol`, o packed as bf16.
@@ -195,19 +188,64 @@ __device__ __forceinline__ void apply_chunk8(const ApplyArgs& ap, int prow, int 
     }
 }
 
+// The addend: the lane that owns row (a*32 + lr) needs columns b*32 + 8q + 4g .. +4 of it.  Fetched
+// that way from global memory, every load instruction would touch 32 different rows for 16 bytes
+// each and the address pipe would take longer than the whole rest of the epilogue.  So the wave's
+// WM x 64 piece of D is first streamed into its staging area `stage_d` (WM rows of 128 bytes) by
+// the DMA path, one instruction per 8 full rows (chunks XOR-swizzled as in the operand ring), and
+// the row-owning 8-byte pieces are read from LDS.  All of them are in registers when this returns:
+// before any store of the sub-tile (D may alias C: in-place a*X + B*X).
+template <int WGN, int WM, int WN, int TM, int TN>
+__device__ __forceinline__ void ns_epilogue_addend(u32x2 (&dv)[TM][TN][4], const MuonGemmDesc& d,
+                                                   const MuonTileJob& job, const char* stage_d) {
+    static_assert(WN == 64, "the addend staging assumes 128-byte rows");
+    int tid_e = threadIdx.x;
+    asm volatile("" : "+v"(tid_e));            // see ns_epilogue_strips
+    const int lane = tid_e & 63, wave = __builtin_amdgcn_readfirstlane(tid_e >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lr = lane & 31, g = lane >> 5;
+    const int row0 = job.i0 + wm * WM, col0 = job.j0 + wn * WN;
+    const uint32_t stage_lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(
+        reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)stage_d)));
+    const int drow = lane >> 3;                         // row within the 8 rows of one instruction
+#pragma unroll
+    for (int j = 0; j < WM / 8; ++j) {
+        const int rr = j * 8 + drow;
+        const int lc = (lane & 7) ^ ((rr >> 1) & 7);    // logical 16-byte chunk this lane fetches
+        dma16(d.D + static_cast<size_t>(row0 + rr) * d.ldd + col0 + lc * 8, stage_lds + j * 1024);
+    }
+    NS_WAIT_VMCNT(0);
+#pragma unroll
+    for (int a = 0; a < TM; ++a) {
+        const int rr = a * 32 + lr;
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                dv[a][b][q] = *reinterpret_cast<const u32x2*>(
+                    stage_d + rr * 128 + (((b * 4 + q) ^ ((rr >> 1) & 7)) * 16) + g * 8);
+    }
+}
+
+// Wave-private staging bytes of the result strips: one 32-row strip in the direct orientation, then
+// (in the same place) the strip's WN rows of 32 columns in the transposed one; rows padded by 16 B.
+constexpr int strip_stage_bytes(int WN) {
+    return 32 * (WN * 2 + 16) > WN * (32 * 2 + 16) ? 32 * (WN * 2 + 16) : WN * (32 * 2 + 16);
+}
+
 // Per 32-row strip of the wave's sub-tile, per 32 x 32 tile of it: t1 = alpha*acc -> row-owning
 // layout -> + beta*D -> o (bf16) -> staged row-major in LDS -> 16-byte coalesced stores of C (and
 // gamma*o to C2); o moved back to the column-owning layout -> staged -> 16-byte coalesced stores
 // of CT (and C2T).  With APPLY, the orientation of the parameter goes through the fused parameter
-// step instead of a store, and the other orientation is not produced.
+// step instead of a store, and the other orientation is not produced.  `stage` is this wave's
+// strip_stage_bytes(WN) of LDS.
 template <bool HAS_D, bool STREAM, bool APPLY, int WGN, int WM, int WN, int TM, int TN>
-__device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const MuonGemmDesc& d,
-                                                 const MuonTileJob& job, float alpha, float beta,
-                                                 float gamma, bool round_terms, char* stage,
-                                                 const ApplyArgs& ap) {
+__device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const u32x2 (&dv)[TM][TN][4],
+                                                   const MuonGemmDesc& d, const MuonTileJob& job, float alpha,
+                                                   float beta, float gamma, bool round_terms, char* stage,
+                                                   const ApplyArgs& ap) {
     constexpr int DROW = WN * 2 + 16;   // staged row pitch in bytes, direct orientation (32 rows)
     constexpr int TROW = 32 * 2 + 16;   // transposed orientation (WN rows of one strip's 32 columns)
-    constexpr int TOFF = 32 * DROW;     // the transposed strip sits behind the direct one
     // The thread index goes through an opaque move here: everything the epilogue derives from it
     // is then computed after the main loop instead of being hoisted above it, where it would sit
     // in registers the loop needs (and be spilled to scratch memory by every wave).
@@ -228,41 +266,6 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
         const int rho = 8 * (t >> 2) + 4 * g + (t & 3);
         id0[t] = static_cast<__bf16>(rho == lr ? 1.0f : 0.0f);
         id1[t] = static_cast<__bf16>(16 + rho == lr ? 1.0f : 0.0f);
-    }
-
-    // addend: the lane that owns row (a*32 + lr) needs columns b*32 + 8q + 4g .. +4 of it.  Fetched
-    // that way from global memory, every load instruction would touch 32 different rows for 16
-    // bytes each and the address pipe would take longer than the whole rest of the epilogue.  So
-    // the wave's WM x 64 piece of D is first streamed into its staging area by the DMA path, one
-    // instruction per 8 full rows (chunks XOR-swizzled as in the operand ring), and the
-    // row-owning 8-byte pieces are read from LDS.  All of them are in registers before the
-    // staging area is reused for the results, and before any store of this sub-tile (D may alias
-    // C: in-place a*X + B*X).
-    static_assert(WN == 64, "the addend staging assumes 128-byte rows");
-    u32x2 dv[TM][TN][4];
-    if (HAS_D) {
-        const uint32_t stage_lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(
-            reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)stage)));
-        const int drow = lane >> 3;                         // row within the 8 rows of one instruction
-#pragma unroll
-        for (int j = 0; j < WM / 8; ++j) {
-            const int rr = j * 8 + drow;
-            const int lc = (lane & 7) ^ ((rr >> 1) & 7);    // logical 16-byte chunk this lane fetches
-            dma16(d.D + static_cast<size_t>(row0 + rr) * d.ldd + col0 + lc * 8, stage_lds + j * 1024);
-        }
-        NS_WAIT_VMCNT(0);
-#pragma unroll
-        for (int a = 0; a < TM; ++a) {
-            const int rr = a * 32 + lr;
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    dv[a][b][q] = *reinterpret_cast<const u32x2*>(
-                        stage + rr * 128 + (((b * 4 + q) ^ ((rr >> 1) & 7)) * 16) + g * 8);
-        }
-        // (a wave's LDS operations execute in order: these reads are done before the results
-        // below overwrite the area)
     }
 
 #pragma unroll
@@ -349,7 +352,7 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
                     u32x2 pk;
                     pk.x = ot[b][2 * q];
                     pk.y = ot[b][2 * q + 1];
-                    *reinterpret_cast<u32x2*>(stage + TOFF + (b * 32 + lr) * TROW + (8 * q + 4 * g) * 2) = pk;
+                    *reinterpret_cast<u32x2*>(stage + (b * 32 + lr) * TROW + (8 * q + 4 * g) * 2) = pk;
                 }
             constexpr int CPR = 32 / 8, RPI = 64 / CPR;
             const int r = lane / CPR, ch = lane % CPR;
@@ -357,14 +360,14 @@ __device__ __forceinline__ void ns_epilogue_impl(f32x16 (&acc)[TM][TN], const Mu
 #pragma unroll 1
                 for (int it = 0; it < WN / RPI; ++it) {
                     const int row = it * RPI + r;
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + TOFF + row * TROW + ch * 16);
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
                     apply_chunk8(ap, col0 + row, row0 + a * 32 + ch * 8, v);
                 }
             } else {
 #pragma unroll
                 for (int it = 0; it < WN / RPI; ++it) {
                     const int row = it * RPI + r;
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + TOFF + row * TROW + ch * 16);
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + row * TROW + ch * 16);
                     const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + a * 32 + ch * 8;
                     gstore16<STREAM>(d.CT + off, v);
                     if (d.C2T) gstore16<STREAM>(d.C2T + off, scale_bf16x8(v, gamma));
@@ -399,8 +402,17 @@ struct GemmCfg {
     static constexpr int HALF_BYTES = BT_ * ROW_BYTES;
     static constexpr int DPH = BT_ / 8 / NW;          // DMA instructions (8 rows each) per wave per half
     static constexpr size_t RING_BYTES = static_cast<size_t>(NHALF) * HALF_BYTES;
-    static constexpr size_t EPI_BYTES = static_cast<size_t>(NW) * epilogue_stage_bytes(WM, WN);
-    static constexpr size_t LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
+    static constexpr size_t LDS_BYTES = RING_BYTES;
+    // After the main loop the ring is free.  The addend pieces (WM rows of 128 bytes per wave) are
+    // staged at its start; once they are in registers, the first NPRE half-stages of the
+    // workgroup's next job are fetched into slots 0 .. NPRE-1 while the result strips are staged
+    // behind them.
+    static constexpr int NPRE = 3;
+    static constexpr size_t ADDEND_BYTES = static_cast<size_t>(NW) * WM * 128;
+    static constexpr size_t STRIP_OFFSET = static_cast<size_t>(NPRE) * HALF_BYTES;
+    static constexpr size_t STRIP_BYTES = strip_stage_bytes(WN);
+    static_assert(ADDEND_BYTES <= RING_BYTES, "addend staging");
+    static_assert(STRIP_OFFSET + NW * STRIP_BYTES <= RING_BYTES, "strip staging behind the prefetched halves");
     static_assert(BT_ % (8 * NW) == 0, "DMA tiling");
     static_assert((NHALF - 2) * DPH < 64 && NHALF >= 5, "vmcnt immediate / ring depth");
     static_assert(NW % 2 == 0, "swizzle parity assumes an even wave count");
@@ -408,40 +420,53 @@ struct GemmCfg {
     static_assert(LDS_BYTES <= 163840, "LDS capacity of a gfx950 CU");
 };
 
+// A launch is persistent: it has as many workgroups as the GPU holds at once (or one per job when
+// there are fewer jobs), and workgroup b computes jobs b, b + gridDim.x, b + 2 gridDim.x, ... of the
+// list.  Workgroups are dealt round-robin to the XCDs, so with a grid that is a multiple of 8 job j
+// still runs on XCD j % 8, in list order.  Between two jobs of a workgroup nothing waits for a
+// launch: the descriptors of the next job are read while the addend of the current one is in
+// flight, and its first NPRE half-stages stream into LDS while the epilogue of the current one
+// runs.
 // APPLY: the launch is the last update product of the iteration and its epilogue takes the
 // parameter step (mats[job.desc] describes the parameter of the job's matrix; `sc`, when given,
 // holds {lr, wd_factor} in device memory and overrides the by-value arguments).
 template <typename Cfg, bool APPLY>
 __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
-    const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, float alpha,
+    const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, int njobs, float alpha,
     float beta, float gamma, int flags, float* __restrict__ split_partials,
     int32_t* __restrict__ split_counters, const MuonMatDesc* __restrict__ mats, float neg_lr,
     float wd_factor, const float* __restrict__ sc) {
     constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
-    constexpr int NHALF = Cfg::NHALF;
+    constexpr int NHALF = Cfg::NHALF, NPRE = Cfg::NPRE;
     extern __shared__ __align__(16) uint16_t lds[];
-    const MuonTileJob job = jobs[blockIdx.x];
-    const MuonGemmDesc d = descs[job.desc];
-    const int i0 = job.i0, j0 = job.j0;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
+    const int tid = threadIdx.x;
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint16_t*)lds));
 
     // ---- DMA addressing: instruction j of this wave fills half-stage rows (j*NW + wave)*8 .. +8;
     //      lane -> row + lane/8, LDS chunk position lane%8, i.e. global chunk (lane%8) ^ swizzle,
     //      swizzle = (row >> 1) & 7 = 4*(wave & 1) + lane/16 ---------------------------------------
-    const int gchunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
+    // The per-lane constants of the main loop are derived once per job from an opaque copy of the
+    // thread index: they are a few instructions, and kept across the epilogue they would cost it
+    // registers it does not have.
+#define NS_LANE_CONSTANTS()                                                                    \
+    int tid_l = tid;                                                                           \
+    asm volatile("" : "+v"(tid_l));                                                            \
+    const int lane = tid_l & 63, wave = __builtin_amdgcn_readfirstlane(tid_l >> 6);            \
+    const int wm = wave / WGN, wn = wave % WGN;                                                \
+    const int gchunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));                         \
+    const uint32_t dst0 = lds_base + wave * 1024
     const uint16_t* srcp[DPH];
     const uint16_t* srcq[DPH];
-#pragma unroll
-    for (int j = 0; j < DPH; ++j) {
-        const int r = (j * NW + wave) * 8 + (lane >> 3);
-        srcp[j] = d.P + static_cast<size_t>(i0 + r) * d.ldp + job.k0 + gchunk * 8;
-        srcq[j] = d.Q + static_cast<size_t>(j0 + r) * d.ldq + job.k0 + gchunk * 8;
-    }
-    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-        (__attribute__((address_space(3))) uint16_t*)lds));
-    const uint32_t dst0 = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+#define NS_SET_SOURCES(job_, d_)                                                               \
+    do {                                                                                       \
+        _Pragma("unroll") for (int j_ = 0; j_ < DPH; ++j_) {                                   \
+            const int r_ = (j_ * NW + wave) * 8 + (lane >> 3);                                 \
+            srcp[j_] = (d_).P + static_cast<size_t>((job_).i0 + r_) * (d_).ldp + (job_).k0 + gchunk * 8; \
+            srcq[j_] = (d_).Q + static_cast<size_t>((job_).j0 + r_) * (d_).ldq + (job_).k0 + gchunk * 8; \
+        }                                                                                      \
+    } while (0)
 
     // half h = 2*kb (+1): P (Q) rows of k-block kb, into ring slot h % NHALF
 #define NS_ISSUE_HALF(src_, kb_, slot_)                                                        \
@@ -450,46 +475,72 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             dma16(src_[j_] + static_cast<size_t>(kb_) * BK,                                    \
                   dst0 + (slot_) * HALF_BYTES + j_ * NW * 1024);                               \
     } while (0)
-
-    // ---- fragment addressing (bytes): lane l reads row l%32, chunk 2*ks + l/32 -------------
-    const int swz = (lane >> 1) & 7;
-    const int c0 = (lane >> 5) ^ swz;
-    const char* const ldsb = reinterpret_cast<const char*>(lds);
-    const char* const pfrag = ldsb + (wm * WM + (lane & 31)) * ROW_BYTES;
-    const char* const qfrag = ldsb + (wn * WN + (lane & 31)) * ROW_BYTES;
-    const int koff[4] = {c0 * 16, (c0 ^ 2) * 16, (c0 ^ 4) * 16, (c0 ^ 6) * 16};
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
-
-    const int nk = (job.k1 - job.k0) / BK;      // this job's share of the reduction
-    // prologue: halves 0 .. NHALF-1 = P0 Q0 P1 Q1 P2 ...
-#pragma unroll
-    for (int h = 0; h < NHALF; ++h) {
-        if (h < 2 * nk) {
-            if (h & 1) NS_ISSUE_HALF(srcq, h >> 1, h);
-            else NS_ISSUE_HALF(srcp, h >> 1, h);
-        }
-    }
+    // the first halves of a job, h in [H0_, H1_) and below 2*nk_: P0 Q0 P1 Q1 P2 ... into slots 0 1 2 ...
+#define NS_ISSUE_FIRST_HALVES(H0_, H1_, nk_)                                                   \
+    do {                                                                                       \
+        _Pragma("unroll") for (int h_ = (H0_); h_ < (H1_); ++h_) {                             \
+            if (h_ < 2 * (nk_)) {                                                              \
+                if (h_ & 1) NS_ISSUE_HALF(srcq, h_ >> 1, h_);                                  \
+                else NS_ISSUE_HALF(srcp, h_ >> 1, h_);                                         \
+            }                                                                                  \
+        }                                                                                      \
+    } while (0)
 
     constexpr int KSTEPS = BK / 16;
     constexpr int DPK = 2 * DPH / KSTEPS;                    // DMA instructions per k-step
     static_assert(2 * DPH % KSTEPS == 0 && DPH % DPK == 0, "DMA instructions must spread evenly");
     static_assert(DPK <= TM, "one DMA instruction per row of MFMAs");
 
-    // Block 0 has landed once only the younger prologue halves are pending.
-    WaitHalves<DPH, NHALF - 2>::run((2 * nk < NHALF ? 2 * nk : NHALF) - 2);
-    __syncthreads();
+    const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
+    if constexpr (APPLY) {
+        if (sc) {
+            neg_lr = -sc[0];
+            wd_factor = sc[1];
+        }
+    }
 
-    // Fragments are double buffered over k-steps ACROSS blocks: the ds_reads of the next k-step
-    // (the first one of block kb+1 included) are issued ahead of the MFMAs of the current one, so
-    // the matrix pipe never waits for LDS latency, not even right after the barrier.
-    bf16x8 af[2][TM], bfr[2][TN];
+    int job_idx = blockIdx.x;                   // the launcher never starts more workgroups than jobs
+    MuonTileJob job = jobs[job_idx];
+    MuonGemmDesc d = descs[job.desc];
+    int nk = (job.k1 - job.k0) / BK;            // this job's share of the reduction
+    {
+        NS_LANE_CONSTANTS();
+        (void)wm;
+        (void)wn;
+        NS_SET_SOURCES(job, d);
+        NS_ISSUE_FIRST_HALVES(0, NHALF, nk);    // prologue: halves 0 .. NHALF-1
+    }
+
+    for (;;) {
+        NS_LANE_CONSTANTS();
+        // ---- fragment addressing (bytes): lane l reads row l%32, chunk 2*ks + l/32 -------------
+        const int swz = (lane >> 1) & 7;
+        const int c0 = (lane >> 5) ^ swz;
+        const char* const ldsb = reinterpret_cast<const char*>(lds);
+        const char* const pfrag = ldsb + (wm * WM + (lane & 31)) * ROW_BYTES;
+        const char* const qfrag = ldsb + (wn * WN + (lane & 31)) * ROW_BYTES;
+        const int koff[4] = {c0 * 16, (c0 ^ 2) * 16, (c0 ^ 4) * 16, (c0 ^ 6) * 16};
+        // the sources of the halves beyond the first ones (set again: the copies made when the
+        // first halves were issued are not kept across the epilogue before)
+        NS_SET_SOURCES(job, d);
+
+        f32x16 acc[TM][TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+
+        // Block 0 has landed once only the younger first halves are pending (for a job after the
+        // first, halves 0 .. NPRE-1 landed long ago and at most NHALF - NPRE are pending).
+        WaitHalves<DPH, NHALF - 2>::run((2 * nk < NHALF ? 2 * nk : NHALF) - 2);
+        __syncthreads();
+
+        // Fragments are double buffered over k-steps ACROSS blocks: the ds_reads of the next k-step
+        // (the first one of block kb+1 included) are issued ahead of the MFMAs of the current one, so
+        // the matrix pipe never waits for LDS latency, not even right after the barrier.
+        bf16x8 af[2][TM], bfr[2][TN];
 #define NS_LOAD_FRAGS(buf_, pf_, qf_, ks_)                                                      \
     do {                                                                                       \
         _Pragma("unroll") for (int a_ = 0; a_ < TM; ++a_)                                      \
@@ -497,149 +548,223 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         _Pragma("unroll") for (int b_ = 0; b_ < TN; ++b_)                                      \
             bfr[buf_][b_] = *reinterpret_cast<const bf16x8*>((qf_) + b_ * 32 * ROW_BYTES + koff[ks_]); \
     } while (0)
-    NS_LOAD_FRAGS(0, pfrag, qfrag + HALF_BYTES, 0);
+        NS_LOAD_FRAGS(0, pfrag, qfrag + HALF_BYTES, 0);
 
-    // The pair of halves being issued: created at the barrier of block kb (last k-step), its
-    // 2*DPH DMA instructions are spread over that k-step and the first KSTEPS-1 of block kb+1,
-    // one after each of the first DPK rows of MFMAs -- a burst right after the barrier would hold
-    // every wave in the memory-issue queue while the matrix pipe sits idle.
-    // NHALF odd: the first half of a pair is a Q half (needed one block earlier), the second P.
-    const uint16_t* const* dsrc[2] = {(NHALF & 1) ? srcq : srcp, (NHALF & 1) ? srcp : srcq};
-    uint32_t ddst[2] = {0, 0};
-    size_t dk[2] = {0, 0};
-    bool dgo[2] = {false, false};
+        // The pair of halves being issued: created at the barrier of block kb (last k-step), its
+        // 2*DPH DMA instructions are spread over that k-step and the first KSTEPS-1 of block kb+1,
+        // one after each of the first DPK rows of MFMAs -- a burst right after the barrier would hold
+        // every wave in the memory-issue queue while the matrix pipe sits idle.
+        // NHALF odd: the first half of a pair is a Q half (needed one block earlier), the second P.
+        const uint16_t* const* dsrc[2] = {(NHALF & 1) ? srcq : srcp, (NHALF & 1) ? srcp : srcq};
+        uint32_t ddst[2] = {0, 0};
+        size_t dk[2] = {0, 0};
+        bool dgo[2] = {false, false};
 
-    int sp = 0, sq = 1;                 // ring slots of the P and Q halves of block kb
-    for (int kb = 0; kb < nk; ++kb) {
-        const char* const pf = pfrag + sp * HALF_BYTES;
-        const char* const qf = qfrag + sq * HALF_BYTES;
-        int spn = sp + 2; spn = spn >= NHALF ? spn - NHALF : spn;
-        int sqn = sq + 2; sqn = sqn >= NHALF ? sqn - NHALF : sqn;
+        int sp = 0, sq = 1;                 // ring slots of the P and Q halves of block kb
+        for (int kb = 0; kb < nk; ++kb) {
+            const char* const pf = pfrag + sp * HALF_BYTES;
+            const char* const qf = qfrag + sq * HALF_BYTES;
+            int spn = sp + 2; spn = spn >= NHALF ? spn - NHALF : spn;
+            int sqn = sq + 2; sqn = sqn >= NHALF ? sqn - NHALF : sqn;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            const int cur = ks & 1, nxt = cur ^ 1;
-            if (ks + 1 < KSTEPS) {
-                NS_LOAD_FRAGS(nxt, pf, qf, ks + 1);
-            } else if (kb + 1 < nk) {
-                // Every fragment of block kb is in registers (the barrier waits for this wave's
-                // LDS reads).  Block kb+1 has landed once only the younger halves are pending;
-                // after the barrier it is visible to all waves and the two slots of block kb are
-                // free for the next pair of halves, 2kb+NHALF and 2kb+NHALF+1.
-                const int issued = 2 * nk < 2 * kb + NHALF ? 2 * nk : 2 * kb + NHALF;
-                WaitHalves<DPH, NHALF - 2>::run(issued - (2 * kb + 4));
-                __syncthreads();
-                const int h0 = 2 * kb + NHALF;
-                ddst[0] = dst0 + sp * HALF_BYTES;                // h0 % NHALF == 2kb % NHALF
-                ddst[1] = dst0 + sq * HALF_BYTES;
-                dk[0] = static_cast<size_t>(h0 >> 1) * BK;
-                dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;
-                dgo[0] = h0 < 2 * nk;
-                dgo[1] = h0 + 1 < 2 * nk;
-                NS_LOAD_FRAGS(nxt, pfrag + spn * HALF_BYTES, qfrag + sqn * HALF_BYTES, 0);
-            } else {
-                dgo[0] = dgo[1] = false;     // last block: nothing left to fetch
-            }
-            __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
-#pragma unroll
-            for (int a = 0; a < TM; ++a) {
-#pragma unroll
-                for (int b = 0; b < TN; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][a], bfr[cur][b], acc[a][b], 0, 0, 0);
-                if (a < DPK) {
-                    // instruction jj of the current pair: the last k-step starts a pair
-                    const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;
-                    const int h = jj / DPH, j = jj % DPH;
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024);
-                    __builtin_amdgcn_sched_barrier(0);
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                const int cur = ks & 1, nxt = cur ^ 1;
+                if (ks + 1 < KSTEPS) {
+                    NS_LOAD_FRAGS(nxt, pf, qf, ks + 1);
+                } else if (kb + 1 < nk) {
+                    // Every fragment of block kb is in registers (the barrier waits for this wave's
+                    // LDS reads).  Block kb+1 has landed once only the younger halves are pending;
+                    // after the barrier it is visible to all waves and the two slots of block kb are
+                    // free for the next pair of halves, 2kb+NHALF and 2kb+NHALF+1.
+                    const int issued = 2 * nk < 2 * kb + NHALF ? 2 * nk : 2 * kb + NHALF;
+                    WaitHalves<DPH, NHALF - 2>::run(issued - (2 * kb + 4));
+                    __syncthreads();
+                    const int h0 = 2 * kb + NHALF;
+                    ddst[0] = dst0 + sp * HALF_BYTES;                // h0 % NHALF == 2kb % NHALF
+                    ddst[1] = dst0 + sq * HALF_BYTES;
+                    dk[0] = static_cast<size_t>(h0 >> 1) * BK;
+                    dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;
+                    dgo[0] = h0 < 2 * nk;
+                    dgo[1] = h0 + 1 < 2 * nk;
+                    NS_LOAD_FRAGS(nxt, pfrag + spn * HALF_BYTES, qfrag + sqn * HALF_BYTES, 0);
+                } else {
+                    dgo[0] = dgo[1] = false;     // last block: nothing left to fetch
                 }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        sp = spn;
-        sq = sqn;
-    }
-#undef NS_LOAD_FRAGS
-#undef NS_ISSUE_HALF
-    __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
-
-    // ---- split reduction (small tile class only): a tile whose K range is shared by `count`
-    //      jobs.  Each job parks its fp32 accumulators in its own slot; the job that arrives last
-    //      adds the slots in slot order (so the sum does not depend on which job that is) and
-    //      writes the tile.  Nobody waits for anybody: the other jobs just exit.
-    //      Hand-over: the slots are written with device-scope stores, which go through to memory
-    //      past the XCD-private L2; after the workgroup barrier one thread takes the ticket with
-    //      release order at device scope, so every slot store of the workgroup happens before
-    //      the ticket is visible.  Only the one job per tile that adds the slots up pays for an
-    //      acquire fence (which drops what its XCD's L2 holds of them) before its plain loads. ----
-    if constexpr (Cfg::SPLIT_K) {
-        const int split_count = job.split >> 16;
-        if (split_count > 1) {
-            constexpr size_t TILE_ELEMS = static_cast<size_t>(Cfg::BM) * Cfg::BN;
-            float* const mine = split_partials + (static_cast<size_t>(job.part_base) + (job.split & 0xffff)) * TILE_ELEMS;
-            const size_t lane_off = static_cast<size_t>(wave) * TM * TN * 16 * 64 + lane;
-#pragma unroll
-            for (int a = 0; a < TM; ++a)
-#pragma unroll
-                for (int b = 0; b < TN; ++b)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        __hip_atomic_store(&mine[lane_off + ((a * TN + b) * 16 + i) * 64], acc[a][b][i],
-                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_s_waitcnt(0);                     // this wave's slot stores are acknowledged ...
-            __syncthreads();
-            int* const ticket = reinterpret_cast<int*>(lds);
-            if (tid == 0)                                      // ... and the whole slot is out before I am counted
-                *ticket = __hip_atomic_fetch_add(&split_counters[job.part_base], 1, NS_SPLIT_TICKET_ORDER,
-                                                 __HIP_MEMORY_SCOPE_AGENT);
-            __syncthreads();
-            const bool last = *ticket == split_count - 1;
-            __syncthreads();                                   // the ticket is read before LDS is reused
-            if (!last) return;
-            if (tid == 0)                                      // ready for the next launch on the stream
-                __hip_atomic_store(&split_counters[job.part_base], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); // drop what this XCD cached of the slots
-            const float* const first = split_partials + static_cast<size_t>(job.part_base) * TILE_ELEMS;
-#pragma unroll
-            for (int a = 0; a < TM; ++a)
-#pragma unroll
-                for (int b = 0; b < TN; ++b)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
-            // slot by slot, all of a lane's loads of one slot in flight together
-            for (int sidx = 0; sidx < split_count; ++sidx) {
-                const float* const slot = first + sidx * TILE_ELEMS;
+                __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
 #pragma unroll
                 for (int a = 0; a < TM; ++a) {
-                    float t[TN][16];
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][a], bfr[cur][b], acc[a][b], 0, 0, 0);
+                    if (a < DPK) {
+                        // instruction jj of the current pair: the last k-step starts a pair
+                        const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;
+                        const int h = jj / DPH, j = jj % DPH;
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            sp = spn;
+            sq = sqn;
+        }
+#undef NS_LOAD_FRAGS
+        __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
+
+        const int next_idx = job_idx + static_cast<int>(gridDim.x);
+        const bool has_next = next_idx < njobs;
+
+        // ---- split reduction (small tile class only): a tile whose K range is shared by `count`
+        //      jobs.  Each job parks its fp32 accumulators in its own slot; the job that arrives last
+        //      adds the slots in slot order (so the sum does not depend on which job that is) and
+        //      writes the tile.  Nobody waits for anybody: the other jobs go on to their next job.
+        //      Hand-over: the slots are written with device-scope stores, which go through to memory
+        //      past the XCD-private L2; after the workgroup barrier one thread takes the ticket with
+        //      release order at device scope, so every slot store of the workgroup happens before
+        //      the ticket is visible.  Only the one job per tile that adds the slots up pays for an
+        //      acquire fence (which drops what its XCD's L2 holds of them) before its plain loads. ----
+        bool write_tile = true;
+        if constexpr (Cfg::SPLIT_K) {
+            const int split_count = job.split >> 16;
+            if (split_count > 1) {
+                constexpr size_t TILE_ELEMS = static_cast<size_t>(Cfg::BM) * Cfg::BN;
+                float* const mine = split_partials + (static_cast<size_t>(job.part_base) + (job.split & 0xffff)) * TILE_ELEMS;
+                // (opaque, so that the 64 slot addresses derived from it are not hoisted out of the
+                // job loop and carried in registers through the main loop)
+                int tid_s = tid;
+                asm volatile("" : "+v"(tid_s));
+                const size_t lane_off = static_cast<size_t>(tid_s >> 6) * TM * TN * 16 * 64 + (tid_s & 63);
+#pragma unroll
+                for (int a = 0; a < TM; ++a)
 #pragma unroll
                     for (int b = 0; b < TN; ++b)
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) t[b][i] = slot[lane_off + ((a * TN + b) * 16 + i) * 64];
-                    __builtin_amdgcn_sched_barrier(0);     // all of these loads go out before the first add waits
+                        for (int i = 0; i < 16; ++i)
+                            __hip_atomic_store(&mine[lane_off + ((a * TN + b) * 16 + i) * 64], acc[a][b][i],
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_s_waitcnt(0);                     // this wave's slot stores are acknowledged ...
+                __syncthreads();
+                int* const ticket = reinterpret_cast<int*>(lds);
+                if (tid == 0)                                      // ... and the whole slot is out before I am counted
+                    *ticket = __hip_atomic_fetch_add(&split_counters[job.part_base], 1, NS_SPLIT_TICKET_ORDER,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                const bool last = *ticket == split_count - 1;
+                __syncthreads();                                   // the ticket is read before LDS is reused
+                write_tile = last;
+                if (last) {
+                    if (tid == 0)                                  // ready for the next launch on the stream
+                        __hip_atomic_store(&split_counters[job.part_base], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); // drop what this XCD cached of the slots
+                    const float* const first = split_partials + static_cast<size_t>(job.part_base) * TILE_ELEMS;
 #pragma unroll
-                    for (int b = 0; b < TN; ++b)
+                    for (int a = 0; a < TM; ++a)
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) acc[a][b][i] += t[b][i];
-                    __builtin_amdgcn_sched_barrier(0);
+                        for (int b = 0; b < TN; ++b)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+                    // slot by slot, all of a lane's loads of one slot in flight together
+                    for (int sidx = 0; sidx < split_count; ++sidx) {
+                        const float* const slot = first + sidx * TILE_ELEMS;
+#pragma unroll
+                        for (int a = 0; a < TM; ++a) {
+                            float t[TN][16];
+#pragma unroll
+                            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                                for (int i = 0; i < 16; ++i) t[b][i] = slot[lane_off + ((a * TN + b) * 16 + i) * 64];
+                            __builtin_amdgcn_sched_barrier(0);     // all of these loads go out before the first add waits
+#pragma unroll
+                            for (int b = 0; b < TN; ++b)
+#pragma unroll
+                                for (int i = 0; i < 16; ++i) acc[a][b][i] += t[b][i];
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
                 }
             }
         }
+
+        // ---- epilogue, first part: the addend into registers (staged at the start of the ring) ----
+        const bool has_d = APPLY || d.D != nullptr;
+        u32x2 dv[TM][TN][4];
+        if (write_tile && has_d) {
+            ns_epilogue_addend<WGN, WM, WN, TM, TN>(dv, d, job, reinterpret_cast<const char*>(lds) + wave * (WM * 128));
+        } else {
+            // defined on every path, so that nothing of it is carried around the job loop in registers
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) dv[a][b][q] = u32x2{0u, 0u};
+        }
+
+        // ---- the next job's first half-stages stream in while the result strips are written -----
+        // every wave holds its addend: the start of the ring is free for the next job's halves, and
+        // the part of it under the strip staging of other waves may be overwritten
+        if (write_tile && has_d) __syncthreads();
+
+        // ---- the workgroup's next job: its first half-stages stream in while the result strips
+        //      are written (its descriptors are read again after the strips rather than kept in
+        //      registers across them) ------------------------------------------------------------
+        if (has_next) {
+            const MuonTileJob nj = jobs[next_idx];
+            const MuonGemmDesc nd = descs[nj.desc];
+            const int nnk = (nj.k1 - nj.k0) / BK;
+            NS_SET_SOURCES(nj, nd);
+            NS_ISSUE_FIRST_HALVES(0, NPRE, nnk);
+        }
+        const int wave_e = wave;      // (scalar) for the staging offsets below
+
+        // ---- epilogue, second part: the result strips (staged behind the prefetched halves) ---------
+        if (write_tile) {
+            char* const stage = reinterpret_cast<char*>(lds) + Cfg::STRIP_OFFSET + wave_e * Cfg::STRIP_BYTES;
+            ApplyArgs ap{nullptr, 0.f, 1.f, false};
+            if constexpr (APPLY) {
+                ap.mat = mats + job.desc;
+                ap.neg_lr = neg_lr;
+                ap.wd_factor = wd_factor;
+                ap.vec_ok = (ap.mat->cols % 8 == 0) && ((reinterpret_cast<uintptr_t>(ap.mat->param) & 15) == 0) &&
+                            ((reinterpret_cast<uintptr_t>(ap.mat->out) & 15) == 0);
+                ns_epilogue_strips<true, Cfg::STREAM_STORES, true, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+            } else {
+                if (has_d) ns_epilogue_strips<true, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+                else ns_epilogue_strips<false, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+            }
+        }
+        if (!has_next) break;
+
+        // The next job becomes the current one.  The index goes through an opaque move so that the
+        // descriptors are loaded afresh (from the scalar cache) instead of living in registers
+        // through the epilogue above.
+        int idx = next_idx;
+        asm volatile("" : "+s"(idx));
+        job = jobs[idx];
+        d = descs[job.desc];
+        nk = (job.k1 - job.k0) / BK;
+        {
+            int tid_n = tid;
+            asm volatile("" : "+v"(tid_n));
+            const int lane = tid_n & 63, wave = __builtin_amdgcn_readfirstlane(tid_n >> 6);
+            const int gchunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
+            const uint32_t dst0 = lds_base + wave * 1024;
+            NS_SET_SOURCES(job, d);
+        // The strips of every wave are out of LDS (the stores that read them have been issued from
+        // registers) and, with vmcnt at zero, the prefetched halves have landed: the rest of the
+        // ring can take the remaining first halves, and the wait at the top of the loop sees only those.
+            NS_WAIT_VMCNT(0);
+            __syncthreads();
+            NS_ISSUE_FIRST_HALVES(NPRE, NHALF, nk);
+        }
+        job_idx = idx;
     }
-    char* const stage = reinterpret_cast<char*>(lds) + wave * epilogue_stage_bytes(WM, WN);
-    const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
-    ApplyArgs ap{nullptr, 0.f, 1.f, false};
-    if constexpr (APPLY) {
-        ap.mat = mats + job.desc;
-        ap.neg_lr = sc ? -sc[0] : neg_lr;
-        ap.wd_factor = sc ? sc[1] : wd_factor;
-        ap.vec_ok = (ap.mat->cols % 8 == 0) && ((reinterpret_cast<uintptr_t>(ap.mat->param) & 15) == 0) &&
-                    ((reinterpret_cast<uintptr_t>(ap.mat->out) & 15) == 0);
-        ns_epilogue_impl<true, Cfg::STREAM_STORES, true, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
-    } else {
-        if (d.D) ns_epilogue_impl<true, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
-        else ns_epilogue_impl<false, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, d, job, alpha, beta, gamma, round_terms, stage, ap);
-    }
+#undef NS_ISSUE_FIRST_HALVES
+#undef NS_ISSUE_HALF
+#undef NS_SET_SOURCES
+#undef NS_LANE_CONSTANTS
 }
 
 // Tile classes: square output tile, waves, workgroups per CU.
@@ -682,6 +807,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 struct DeviceState {
     bool ready = false;
+    int num_cus = 0;                          // a persistent launch has num_cus * MINB workgroups at most
     unsigned char* scratch_ptr = nullptr;     // device address of `scratch` on this device
 };
 static DeviceState g_devices[kMaxDevices];
@@ -731,6 +857,7 @@ static int device_setup(const DeviceState** out) {
             return MUON_AMD_ELAUNCH;
         }
         st.scratch_ptr = static_cast<unsigned char*>(ptr);
+        st.num_cus = prop.multiProcessorCount;
         st.ready = true;
     }
     *out = &st;
@@ -744,26 +871,30 @@ struct ApplyLaunch {            // the fused parameter step of the last update p
 };
 
 template <typename Cfg>
-static int launch_gemm(const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs, float alpha,
-                       float beta, float gamma, int flags, float* split_partials,
+static int launch_gemm(const DeviceState& st, const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs,
+                       float alpha, float beta, float gamma, int flags, float* split_partials,
                        int32_t* split_counters, const ApplyLaunch& ap, hipStream_t s) {
+    // as many workgroups as the GPU holds at once; each walks its share of the job list
+    const int resident = st.num_cus * Cfg::MINB;
+    const int grid = njobs < resident ? njobs : resident;
     if (ap.mats)
-        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, true>), dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
-                           alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, true>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                           njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
                            ap.wd_factor, ap.scalars);
     else
-        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false>), dim3(njobs), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
-                           alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                           njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
                            ap.wd_factor, ap.scalars);
     return check_launch("ns_gemm");
 }
 
-static int launch_gemm_class(int tile_class, const MuonGemmDesc* descs, const MuonTileJob* jobs, int njobs,
-                             float alpha, float beta, float gamma, int flags, float* split_partials,
-                             int32_t* split_counters, const ApplyLaunch& ap, hipStream_t s) {
+static int launch_gemm_class(const DeviceState& st, int tile_class, const MuonGemmDesc* descs,
+                             const MuonTileJob* jobs, int njobs, float alpha, float beta, float gamma,
+                             int flags, float* split_partials, int32_t* split_counters, const ApplyLaunch& ap,
+                             hipStream_t s) {
     if (tile_class == 0)
-        return launch_gemm<Cfg0>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
-    return launch_gemm<Cfg1>(descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
+        return launch_gemm<Cfg0>(st, descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
+    return launch_gemm<Cfg1>(st, descs, jobs, njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap, s);
 }
 
 __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, int n) {
@@ -867,7 +998,7 @@ int muon_amd_ns_gemm(const MuonGemmDesc* descs_dev, const MuonTileJob* jobs_dev,
     const DeviceState* st = nullptr;
     const int rc = device_setup(&st);
     if (rc != MUON_AMD_OK) return rc;
-    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
+    return launch_gemm_class(*st, tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
                              split_partials_dev, split_counters_dev, ApplyLaunch{nullptr, 0.f, 1.f, nullptr},
                              static_cast<hipStream_t>(stream));
 }
@@ -882,7 +1013,7 @@ int muon_amd_ns_gemm_apply(const MuonGemmDesc* descs_dev, const MuonTileJob* job
     const DeviceState* st = nullptr;
     const int rc = device_setup(&st);
     if (rc != MUON_AMD_OK) return rc;
-    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, 0.f, flags, nullptr, nullptr,
+    return launch_gemm_class(*st, tile_class, descs_dev, jobs_dev, njobs, alpha, beta, 0.f, flags, nullptr, nullptr,
                              ApplyLaunch{mats_dev, -lr, wd_factor, scalars_dev}, static_cast<hipStream_t>(stream));
 }
 
@@ -913,7 +1044,7 @@ int muon_amd_ns_gemm_noalloc(const MuonGemmDesc* descs_dev, const MuonTileJob* j
         const int zrc = check_launch("ns_gemm_noalloc: clear counters");
         if (zrc != MUON_AMD_OK) return zrc;
     }
-    return launch_gemm_class(tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
+    return launch_gemm_class(*st, tile_class, descs_dev, jobs_dev, njobs, alpha, beta, gamma, flags,
                              split_slots > 0 ? partials : nullptr, split_slots > 0 ? counters : nullptr,
                              ApplyLaunch{nullptr, 0.f, 1.f, nullptr}, s);
 }
