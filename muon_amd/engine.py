@@ -203,18 +203,20 @@ class _ChunkRuntime:
 class MuonGroupEngine:
     """Runs the Muon update of a fixed list of matrix shapes on one device.
 
-    Built once per (shapes, steps, rounding); each `run` takes the current tensor addresses.
+    Built once per (shapes, steps, rounding).  A step is `prepare` (bind the current tensor
+    addresses, take the hyper-parameters) followed by `enqueue` (the launches); `run` does both.
+    `enqueue` either passes the hyper-parameters by value or, given the device address of a copy
+    of `scalars()`, lets the kernels read them at run time -- which is what a caller does who
+    records the launches into a HIP graph once and replays them with new values.
     """
 
+    N_SCALARS = 4          # {1 - beta, beta, lr, 1 - lr * weight_decay}
+
     def __init__(self, shapes, device, steps: int = 5, reference_rounding: bool = True,
-                 workspace_cap: int | None = None, variant: str = "ns5", use_graph: bool = False):
+                 workspace_cap: int | None = None, variant: str = "ns5"):
         self.device = torch.device(device)
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().muon_amd_init(), "init")
-        self.use_graph = bool(use_graph)
-        self._graph = None
-        self._graph_key = None
-        self._scalars = torch.zeros(4, dtype=torch.float32, device=self.device)
         self.shapes = [(int(r), int(c)) for r, c in shapes]
         cap = DEFAULT_WORKSPACE_CAP if workspace_cap is None else int(workspace_cap)
         self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap, variant)
@@ -223,39 +225,43 @@ class MuonGroupEngine:
         base = self.workspace.data_ptr()
         assert base % 256 == 0
         self.runtimes = [_ChunkRuntime(c, base, self.device) for c in self.chunks]
+        self._hyper = None
 
-    def run(self, grads, momenta, params, outs, scales, src_dtypes, *, beta, nesterov, mutate_grad,
-            eps, lr, weight_decay):
-        """All arguments are per-matrix lists in the order of `shapes` (device addresses or 0)."""
-        one_minus_beta = 1 - beta                      # python double, as muon.py:9
-        wd_factor = 1 - lr * weight_decay              # python double, as muon.py:98
+    def prepare(self, grads, momenta, params, outs, scales, src_dtypes, *, beta, nesterov, mutate_grad,
+                eps, lr, weight_decay):
+        """All list arguments are per matrix in the order of `shapes` (device addresses or 0)."""
         for rt in self.runtimes:
             idx = [lay.index for lay in rt.chunk.layouts]
             rt.bind([grads[i] for i in idx], [momenta[i] for i in idx], [params[i] for i in idx],
                     [outs[i] for i in idx], [scales[i] for i in idx], [src_dtypes[i] for i in idx])
-        if not self.use_graph or PROFILE is not None:
-            for rt in self.runtimes:
-                rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor)
-            return
-        # Graph mode: every launch of the step is recorded once into a HIP graph and replayed.
-        # What changes between steps lives in device memory that the recorded launches read: the
-        # matrix descriptors (tensor addresses; rewritten in place by bind() when one moved) and
-        # the hyper-parameter scalars, refreshed here by a small copy ahead of the replay.
-        _upload(np.array([one_minus_beta, beta, lr, wd_factor], dtype=np.float32), self.device,
-                into=self._scalars.view(torch.uint8))
-        key = (bool(nesterov), bool(mutate_grad), float(eps))
-        if self._graph is None or key != self._graph_key:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                for rt in self.runtimes:
-                    rt.run(one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor,
-                           scalars_ptr=self._scalars.data_ptr())
-            self._graph, self._graph_key = graph, key
-        self._graph.replay()
+        # 1 - beta and 1 - lr * weight_decay are python doubles, as in muon.py:9 and muon.py:98
+        self._hyper = dict(one_minus_beta=1 - beta, beta=beta, nesterov=bool(nesterov),
+                           mutate_grad=bool(mutate_grad), eps=float(eps), lr=lr, wd_factor=1 - lr * weight_decay)
+
+    def scalars(self):
+        h = self._hyper
+        return [h["one_minus_beta"], h["beta"], h["lr"], h["wd_factor"]]
+
+    def structure_key(self):
+        """What a recorded sequence of launches depends on besides device memory."""
+        h = self._hyper
+        return (id(self), h["nesterov"], h["mutate_grad"], h["eps"])
+
+    def enqueue(self, scalars_ptr: int = 0):
+        h = self._hyper
+        for rt in self.runtimes:
+            rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
+                   h["wd_factor"], scalars_ptr=scalars_ptr)
+
+    def run(self, grads, momenta, params, outs, scales, src_dtypes, **hyper):
+        self.prepare(grads, momenta, params, outs, scales, src_dtypes, **hyper)
+        self.enqueue()
 
 
 class AdamGroupEngine:
-    """Fused auxiliary-Adam launch over a fixed list of tensors."""
+    """Fused auxiliary-Adam launch over a fixed list of tensors (prepare / enqueue as above)."""
+
+    N_SCALARS = 7          # {lr, 1 - lr * weight_decay, 1 - beta1, 1 - beta2, eps, 1 - beta1**t, 1 - beta2**t}
 
     def __init__(self, numels, device):
         _lib.load()
@@ -264,11 +270,13 @@ class AdamGroupEngine:
         self.prefix = _plan.adam_block_prefix(self.numels)
         self.nblocks = int(self.prefix[-1])
         self.prefix_dev = _upload(self.prefix, self.device)
-        self.desc_dev = None
+        # one buffer for the descriptors, rewritten in place: recorded launches keep its address
+        self.desc_dev = torch.empty(len(self.numels) * _lib.ADAM_DESC.itemsize, dtype=torch.uint8, device=self.device)
         self.key = None
+        self._hyper = None
 
-    def run(self, params, grads, exp_avgs, exp_avg_sqs, updates, *, lr, weight_decay, betas, eps, step,
-            dtypes=None):
+    def prepare(self, params, grads, exp_avgs, exp_avg_sqs, updates, *, lr, weight_decay, betas, eps, step,
+                dtypes=None):
         dtypes = [_lib.SRC_F32] * len(self.numels) if dtypes is None else list(dtypes)
         key = (tuple(params), tuple(grads), tuple(exp_avgs), tuple(exp_avg_sqs), tuple(updates), tuple(dtypes))
         if key != self.key:
@@ -280,14 +288,65 @@ class AdamGroupEngine:
             d["update"] = updates
             d["numel"] = self.numels
             d["dtype"] = dtypes
-            self.desc_dev = _upload(d, self.device)
+            _upload(d, self.device, into=self.desc_dev)
             self.key = key
+            self.nbytes = sum(n * (14 if t == _lib.SRC_BF16 else 28) for n, t in zip(self.numels, dtypes))
+        # python doubles, as muon.py:105-108 and 257
+        self._hyper = [lr, 1 - lr * weight_decay, 1 - betas[0], 1 - betas[1], eps,
+                       1 - betas[0] ** step, 1 - betas[1] ** step]
+
+    def scalars(self):
+        return list(self._hyper)
+
+    def structure_key(self):
+        return (id(self),)
+
+    def enqueue(self, scalars_ptr: int = 0):
         lib = _lib.load()
-        w1 = 1 - betas[0]                              # python doubles, as muon.py:105-108
-        w2 = 1 - betas[1]
-        bias1 = 1 - betas[0] ** step
-        bias2 = 1 - betas[1] ** step
-        nbytes = sum(n * (14 if t == _lib.SRC_BF16 else 28) for n, t in zip(self.numels, dtypes))
-        _launch("adam", nbytes, lambda: _lib.check(lib.muon_amd_adam(
+        lr, wd_factor, w1, w2, eps, bias1, bias2 = self._hyper
+        _launch("adam", self.nbytes, lambda: _lib.check(lib.muon_amd_adam(
             self.desc_dev.data_ptr(), self.prefix_dev.data_ptr(), len(self.numels), self.nblocks, lr,
-            1 - lr * weight_decay, w1, w2, eps, bias1, bias2, None, _stream_ptr(self.device)), "adam"))
+            wd_factor, w1, w2, eps, bias1, bias2, scalars_ptr or None, _stream_ptr(self.device)), "adam"))
+
+    def run(self, params, grads, exp_avgs, exp_avg_sqs, updates, **hyper):
+        self.prepare(params, grads, exp_avgs, exp_avg_sqs, updates, **hyper)
+        self.enqueue()
+
+
+class StepGraph:
+    """A whole optimizer step on one device as one HIP graph: the launches of every engine of the
+    step are recorded once and replayed afterwards.  What changes between steps is read by the
+    recorded kernels from device memory: tensor addresses from the descriptor tables (rewritten in
+    place by the engines' `prepare` when a tensor moved) and the hyper-parameters (learning rates,
+    decay factors, Adam's bias corrections) from one block of scalars that a small asynchronous
+    copy refreshes ahead of every replay.  No memset node is recorded."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.graph = None
+        self.key = None
+        self.scalars = None
+        self.replays = 0
+
+    def run(self, engines):
+        """`engines`: prepared engines in launch order."""
+        offsets, host = [], []
+        for e in engines:
+            offsets.append(len(host))
+            vals = e.scalars()
+            host += vals + [0.0] * ((-len(vals)) % 4)          # every block 16-byte aligned
+        if self.scalars is None or self.scalars.numel() < len(host):
+            self.scalars = torch.zeros(max(len(host), 16), dtype=torch.float32, device=self.device)
+            self.graph = None                                    # recorded launches hold the old address
+        _upload(np.asarray(host, dtype=np.float32), self.device,
+                into=self.scalars.view(torch.uint8)[: 4 * len(host)])
+        key = tuple(e.structure_key() for e in engines)
+        if self.graph is None or key != self.key:
+            graph = torch.cuda.CUDAGraph()
+            base = self.scalars.data_ptr()
+            with torch.cuda.graph(graph):
+                for e, off in zip(engines, offsets):
+                    e.enqueue(base + 4 * off)
+            self.graph, self.key = graph, key
+        self.graph.replay()
+        self.replays += 1

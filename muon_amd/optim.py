@@ -9,7 +9,8 @@ from __future__ import annotations
 
 import torch
 
-from .engine import AdamGroupEngine, MuonGroupEngine, require_gpu_tensor
+from . import engine as _engine
+from .engine import AdamGroupEngine, MuonGroupEngine, StepGraph, require_gpu_tensor
 from .functional import _rounding_flag, _src_dtype
 
 NS_STEPS = 5          # the reference classes never pass a step count: muon_update's default rules
@@ -35,6 +36,10 @@ class _MuonBase(torch.optim.Optimizer):
         self._workspace_bytes = workspace_bytes
         self._muon_engines = {}
         self._adam_engines = {}
+        self._graphs = {}             # device -> StepGraph (use_graph=True)
+        self._pending = []            # engines prepared by the group loop of the current step, in launch order
+        self._writebacks = []         # (destination, contiguous copy) pairs to copy back after the launches
+        self._keepalive = []          # temporaries whose addresses the pending launches use
 
     _RUNTIME_OPTIONS = ("_ns_rounding", "_mutate_grad", "_workspace_bytes", "_ns_variant", "_use_graph")
 
@@ -125,16 +130,18 @@ class _MuonBase(torch.optim.Optimizer):
         eng = self._muon_engines.get(key)
         if eng is None:
             self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
-            eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes,
-                                  variant=self._ns_variant, use_graph=self._use_graph)
+            with torch.cuda.device(device):
+                eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes,
+                                      variant=self._ns_variant)
             self._muon_engines[key] = eng
+            self._graphs.pop(device, None)        # a recorded step refers to the engine that was replaced
         n = len(shapes)
-        with torch.cuda.device(device):
-            eng.run(grads, moms, ptrs, [0] * n, scales, dtypes,
+        eng.prepare(grads, moms, ptrs, [0] * n, scales, dtypes,
                     beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad,
                     eps=1e-7, lr=group["lr"], weight_decay=group["weight_decay"])
-            for dst, src in writebacks:           # stream ordered after the launches
-                dst.copy_(src)
+        self._pending.append(eng)
+        self._writebacks += writebacks
+        self._keepalive.append(keep)
 
     def _adam_group_step(self, gi, group):
         by_step, writebacks = {}, []
@@ -159,17 +166,40 @@ class _MuonBase(torch.optim.Optimizer):
             if eng is None:
                 eng = AdamGroupEngine([p.numel() for p, _ in items], device)
                 self._adam_engines[key] = eng
-            with torch.cuda.device(device):
-                eng.run([t[0].data_ptr() for _, t in items], [t[1].data_ptr() for _, t in items],
+            eng.prepare([t[0].data_ptr() for _, t in items], [t[1].data_ptr() for _, t in items],
                         [t[2].data_ptr() for _, t in items], [t[3].data_ptr() for _, t in items],
                         [0] * len(items),
                         lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"],
                         eps=group["eps"], step=step, dtypes=[_src_dtype(p) for p, _ in items])
-        for dst, src in writebacks:
-            dst.copy_(src)
+            self._pending.append(eng)
+            self._keepalive.append(items)
+        self._writebacks += writebacks
 
-    @staticmethod
-    def _run_closure(closure):
+    def _launch_pending(self):
+        """Enqueue what the group loop prepared: eagerly, or (use_graph=True) as one recorded graph
+        per device that is replayed every step; then copy back tensors that went through a
+        contiguous copy (stream ordered after the launches)."""
+        try:
+            by_device = {}
+            for eng in self._pending:
+                by_device.setdefault(eng.device, []).append(eng)
+            for device, engines in by_device.items():
+                with torch.cuda.device(device):
+                    if self._use_graph and _engine.PROFILE is None:
+                        graph = self._graphs.get(device)
+                        if graph is None:
+                            graph = self._graphs[device] = StepGraph(device)
+                        graph.run(engines)
+                    else:
+                        for eng in engines:
+                            eng.enqueue()
+            for dst, src in self._writebacks:
+                dst.copy_(src)
+        finally:
+            self._pending, self._writebacks, self._keepalive = [], [], []
+
+    def _run_closure(self, closure):
+        self._pending, self._writebacks, self._keepalive = [], [], []     # nothing left over from a step that raised
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -185,9 +215,9 @@ class SingleDeviceMuon(_MuonBase):
     off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace),
     ns_variant ("ns5": the five-iteration specification muon.py:265-291; "aol4": the
     four-iteration AOL-rescaled variant muon.py:748-799, see zeropower_via_aol4), use_graph
-    (record the launches of a Muon group's step into a HIP graph once and replay it every step;
-    tensor addresses and hyper-parameters are read from device memory, so gradients may be
-    reallocated and learning rates scheduled between steps).
+    (record every launch of a step -- all Muon groups and all Adam groups on a device -- into one
+    HIP graph once and replay it every step; tensor addresses and hyper-parameters are read from
+    device memory, so gradients may be reallocated and learning rates scheduled between steps).
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
@@ -201,6 +231,7 @@ class SingleDeviceMuon(_MuonBase):
         loss = self._run_closure(closure)
         for gi, group in enumerate(self.param_groups):
             self._muon_group_step(gi, group)
+        self._launch_pending()
         return loss
 
 
@@ -258,6 +289,7 @@ class SingleDeviceMuonWithAuxAdam(_MuonBase):
                 self._muon_group_step(gi, group)
             else:
                 self._adam_group_step(gi, group)
+        self._launch_pending()
         return loss
 
 

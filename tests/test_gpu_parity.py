@@ -599,7 +599,34 @@ def test_graph_replay_equals_eager_every_step(M):
             og.zero_grad(set_to_none=True)
             del junk
         eng = next(iter(og._muon_engines.values()))
-        assert eng._graph is not None and (cap is None or len(eng.runtimes) > 1)
+        graph = next(iter(og._graphs.values()))
+        # one recorded graph per device holds the Muon chunks and the Adam launch; it was recorded once
+        assert graph.graph is not None and graph.replays == 5 and len(og._graphs) == 1
+        assert cap is None or len(eng.runtimes) > 1
+
+
+def test_graph_replay_matches_the_oracle(M):
+    """The recorded step (Muon chunks of both tile classes and the Adam launch in one graph, with
+    Adam's bias corrections and the learning rates read from device memory) against the oracle."""
+    muon_shapes, adam_shapes = [(768, 768), (1024, 1280), (256, 576), (16, 8, 3, 3)], [(1000, 64), (64,)]
+    cpu_m, gpu_m = _clone_params(muon_shapes, 0.02, 1331)
+    cpu_a, gpu_a = _clone_params(adam_shapes, 0.02, 1332)
+    mk = lambda cls, pm, pa, **kw: cls([dict(params=pm, use_muon=True, lr=0.02, weight_decay=0.01),
+                                        dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), weight_decay=0.01)], **kw)
+    oc = mk(O.OracleSingleDeviceMuonWithAuxAdam, cpu_m, cpu_a)
+    og = mk(M.SingleDeviceMuonWithAuxAdam, gpu_m, gpu_a, use_graph=True)
+    for step in range(4):
+        for o in (oc, og):
+            o.param_groups[1]["lr"] = 3e-4 * (1 + step)          # a schedule on the Adam group
+        _set_grads(cpu_m + cpu_a, gpu_m + gpu_a, 1e-3)
+        oc.step()
+        og.step()
+        for pc, pg in zip(cpu_m, gpu_m):
+            tol = (TOL_PARAM if pc.ndim == 2 else 3e-3) * (step + 1) ** 0.5      # bf16 noise of k steps adds up like a random walk
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= tol, (tuple(pc.shape), step)
+        for pc, pg in zip(cpu_a, gpu_a):
+            np.testing.assert_allclose(pg.detach().cpu().numpy(), pc.detach().numpy(), rtol=TOL_ADAM, atol=1e-8)
+    assert next(iter(og._graphs.values())).replays == 4 and og.state[gpu_a[0]]["step"] == 4
 
 
 def test_split_reduction_is_deterministic_and_batch_independent(M):
