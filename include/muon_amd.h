@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MUON_AMD_ABI_VERSION 1
+#define MUON_AMD_ABI_VERSION 2
 
 #define MUON_AMD_OK        0
 #define MUON_AMD_EINVAL   (-1)   /* bad argument (null pointer, bad size, misaligned table) */
@@ -38,6 +38,14 @@ extern "C" {
 #define MUON_AMD_ROUND_FUSED     0  /* one bf16 rounding per stored output (closer to fp32) */
 #define MUON_AMD_NORM_UNIT       2  /* muon_amd_norm_finalize only: denom = 1 (no Frobenius
                                        pre-scale; the AOL variant rescales by rows instead) */
+#define MUON_AMD_GEMM_ROWSUM     4  /* muon_amd_ns_gemm only, for a mirrored product without addend
+                                       (A = X X^T): also leave, per row of the result, partial sums
+                                       of |A_ij| in MuonGemmDesc.rowsum (muon.py:779-781 fused into
+                                       the product's epilogue) */
+
+/* How muon_amd_aol_rescale scales the Gram matrix (mode argument). */
+#define MUON_AMD_AOL_SYMMETRIC   0  /* A <- diag(r) A diag(r): the Gram matrix of the rescaled X   */
+#define MUON_AMD_AOL_ROWS_ONLY   1  /* A <- diag(r)^2 A = A / s, rows only, as muon.py:785 writes it */
 
 /* Storage type of the caller's tensors of one matrix / Adam tensor: gradient, optimizer state and
  * parameter share it, as they do in the reference (state is zeros_like(p), muon.py:95-96,
@@ -98,6 +106,12 @@ typedef struct MuonGemmDesc {
     int32_t ldp, ldq, ldd, ldc, ldct;   /* leading dimensions in elements, multiples of 8     */
     int32_t K;                          /* multiple of 64                                     */
     int32_t rows, colsn;                /* padded extent of the output (multiples of the tile) */
+    /* MUON_AMD_GEMM_ROWSUM: rows x ld_rowsum floats; entry [i][s] receives the sum of |o_ij| over
+     * the 64 columns j of slot s (every entry with s < colsn / 64 is written exactly once per
+     * launch, some with zero; adding a row's entries in slot order gives sum_j |o_ij|).       */
+    float*  rowsum;
+    int32_t ld_rowsum;                  /* >= colsn / 64                                       */
+    int32_t reserved;                   /* 0                                                   */
 } MuonGemmDesc;
 
 /* One output tile of one matrix, or one share of its reduction.  A tile whose K is long and
@@ -134,7 +148,9 @@ typedef struct MuonAolDesc {
     uint16_t* xc;     /* n_p x m_p bf16 (ld_m): X^T, scaled by r along columns                  */
     uint16_t* gram;   /* m_p x m_p bf16 (ld_m): A = X X^T, becomes diag(r) A diag(r)            */
     float*    rvec;   /* m_p floats: r_i = max(sum_j |A_ij|, eps)^-1/2                          */
+    const float* rowsum; /* m_p x ld_rowsum partial row sums left by the X X^T launch, or NULL      */
     int32_t   m_p, n_p, ld_n, ld_m;
+    int32_t   ld_rowsum, reserved;
 } MuonAolDesc;
 
 int         muon_amd_abi_version(void);
@@ -255,15 +271,22 @@ int muon_amd_aol_rows_per_block(void);
  * Gram matrix, seg_prefix_host[3*nmat+1] over the rows of X, X^T and A of each matrix.        */
 int muon_amd_validate_aol(const MuonAolDesc* descs_host, int nmat, const int32_t* row_prefix_host,
                           const int32_t* seg_prefix_host);
-/* rvec_i = max(bf16(sum_j |A_ij|), eps)^-1/2 for every row of every Gram matrix.             */
+/* rvec_i = max(bf16(sum_j |A_ij|), eps)^-1/2 for every row of every Gram matrix, from a pass
+ * over the stored A.                                                                          */
 int muon_amd_aol_rowsum(const MuonAolDesc* descs_dev, const int32_t* row_prefix_dev, int nmat,
                         int nblocks, float eps, void* stream);
-/* X <- diag(r) X in both stored orientations and A <- diag(r) A diag(r), in place.  The
- * reference divides the rows of A by s = r^-2 instead (muon.py:785), which is not symmetric
- * and, stored through its mirroring kernel, depends on the tile the autotuner picked; the
- * symmetric form is the Gram matrix of the rescaled X that the iteration assumes.            */
+/* The same from the partial row sums that the X X^T launch left under MUON_AMD_GEMM_ROWSUM
+ * (MuonAolDesc.rowsum): no pass over A.  The slots of a row are added in a fixed order.       */
+int muon_amd_aol_rowsum_finalize(const MuonAolDesc* descs_dev, const int32_t* row_prefix_dev, int nmat,
+                                 int nblocks, float eps, void* stream);
+/* X <- diag(r) X in both stored orientations, in place, and the Gram matrix rescaled in place:
+ * MUON_AMD_AOL_SYMMETRIC  A <- diag(r) A diag(r), the Gram matrix of the rescaled X that the
+ *                         iteration assumes;
+ * MUON_AMD_AOL_ROWS_ONLY  A <- A / s (s = r^-2) by rows only, as muon.py:785 writes it: A is
+ *                         then no longer symmetric, and the polynomial launch that follows must
+ *                         cover every tile (no mirrored store).                               */
 int muon_amd_aol_rescale(const MuonAolDesc* descs_dev, const int32_t* seg_prefix_dev, int nmat,
-                         int nblocks, void* stream);
+                         int nblocks, int mode, void* stream);
 
 /* ---- auxiliary Adam (muon.py:104-109 and 255-258) ---------------------------------------- */
 /* m <- lerp(m, g, w1); v <- lerp(v, g*g, w2)  with w1 = 1-beta1, w2 = 1-beta2;

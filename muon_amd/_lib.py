@@ -14,10 +14,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MUON_AMD_LIBRARY: path of another build of the library (for comparing builds side by side)
 LIB_PATH = os.environ.get("MUON_AMD_LIBRARY") or os.path.join(_HERE, "libmuon_amd.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 ROUND_REFERENCE = 1
 ROUND_FUSED = 0
 NORM_UNIT = 2
+GEMM_ROWSUM = 4
+AOL_SYMMETRIC = 0
+AOL_ROWS_ONLY = 1
 SRC_F32 = 0
 SRC_BF16 = 1
 
@@ -32,7 +35,8 @@ MAT_DESC = np.dtype(
 GEMM_DESC = np.dtype(
     [("P", "<u8"), ("Q", "<u8"), ("D", "<u8"), ("C", "<u8"), ("CT", "<u8"), ("C2", "<u8"),
      ("C2T", "<u8"), ("ldp", "<i4"), ("ldq", "<i4"), ("ldd", "<i4"), ("ldc", "<i4"),
-     ("ldct", "<i4"), ("K", "<i4"), ("rows", "<i4"), ("colsn", "<i4")],
+     ("ldct", "<i4"), ("K", "<i4"), ("rows", "<i4"), ("colsn", "<i4"),
+     ("rowsum", "<u8"), ("ld_rowsum", "<i4"), ("reserved", "<i4")],
     align=True)
 TILE_JOB = np.dtype([("desc", "<i4"), ("i0", "<i4"), ("j0", "<i4"), ("diag", "<i4"), ("k0", "<i4"),
                      ("k1", "<i4"), ("part_base", "<i4"), ("split", "<i4")], align=True)
@@ -42,8 +46,8 @@ ADAM_DESC = np.dtype(
     align=True)
 
 AOL_DESC = np.dtype(
-    [("xr", "<u8"), ("xc", "<u8"), ("gram", "<u8"), ("rvec", "<u8"),
-     ("m_p", "<i4"), ("n_p", "<i4"), ("ld_n", "<i4"), ("ld_m", "<i4")],
+    [("xr", "<u8"), ("xc", "<u8"), ("gram", "<u8"), ("rvec", "<u8"), ("rowsum", "<u8"),
+     ("m_p", "<i4"), ("n_p", "<i4"), ("ld_n", "<i4"), ("ld_m", "<i4"), ("ld_rowsum", "<i4"), ("reserved", "<i4")],
     align=True)
 
 _c_int = ctypes.c_int
@@ -63,7 +67,8 @@ SIGNATURES = {
     "muon_amd_aol_rows_per_block": (_c_int, []),
     "muon_amd_validate_aol": (_c_int, [_vp, _c_int, _vp, _vp]),
     "muon_amd_aol_rowsum": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _vp]),
-    "muon_amd_aol_rescale": (_c_int, [_vp, _vp, _c_int, _c_int, _vp]),
+    "muon_amd_aol_rowsum_finalize": (_c_int, [_vp, _vp, _c_int, _c_int, _c_float, _vp]),
+    "muon_amd_aol_rescale": (_c_int, [_vp, _vp, _c_int, _c_int, _c_int, _vp]),
     "muon_amd_elementwise_block_elems": (_c_int, []),
     "muon_amd_normalize_tile": (_c_int, []),
     "muon_amd_gemm_tile_rows": (_c_int, [_c_int]),

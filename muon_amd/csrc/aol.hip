@@ -44,10 +44,28 @@ __global__ __launch_bounds__(AOL_THREADS) void aol_rowsum_kernel(
     if (lane == 0) d.rvec[row] = rsqrtf(fmaxf(round_bf(s), eps));
 }
 
+// The same r from the partial row sums that the X X^T launch left (one float per row and 64-column
+// slot, MUON_AMD_GEMM_ROWSUM): lane l adds slots l, l + 64, ... in order, then the wavefront's
+// butterfly adds the lanes -- a fixed order, whatever else the launch holds.
+__global__ __launch_bounds__(AOL_THREADS) void aol_rowsum_finalize_kernel(
+    const MuonAolDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, float eps) {
+    const int b = blockIdx.x;
+    const int mi = find_segment(prefix, nmat, b);
+    const MuonAolDesc d = descs[mi];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = (b - prefix[mi]) * AOL_ROWS_PER_BLOCK + wave;      // < m_p by construction
+    const float* __restrict__ parts = d.rowsum + static_cast<int64_t>(row) * d.ld_rowsum;
+    float s = 0.f;
+    for (int c = lane; c < d.m_p / 64; c += 64) s += parts[c];
+    s = wave_sum(s);
+    if (lane == 0) d.rvec[row] = rsqrtf(fmaxf(round_bf(s), eps));
+}
+
 // Scales one row of one of the three buffers of a matrix.  Segment 3*mi + 0: rows of X (factor
 // r_row), + 1: rows of X^T (factor r_col), + 2: rows of A (factor r_row * r_col).
+// rows_only: the rows of A take r_row^2 (A / s, muon.py:785) instead of r_row * r_col.
 __global__ __launch_bounds__(AOL_THREADS) void aol_rescale_kernel(
-    const MuonAolDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat) {
+    const MuonAolDesc* __restrict__ descs, const int32_t* __restrict__ prefix, int nmat, int rows_only) {
     const int b = blockIdx.x;
     const int seg = find_segment(prefix, 3 * nmat, b);
     const int mi = seg / 3, kind = seg - 3 * mi;
@@ -74,6 +92,9 @@ __global__ __launch_bounds__(AOL_THREADS) void aol_rescale_kernel(
         if (kind == 0) {
 #pragma unroll
             for (int k = 0; k < 8; ++k) f[k] = r_row;
+        } else if (kind == 2 && rows_only) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) f[k] = r_row * r_row;
         } else {
             const f32x4a r0 = *(const __attribute__((address_space(1))) f32x4a*)(r + c);
             const f32x4a r1 = *(const __attribute__((address_space(1))) f32x4a*)(r + c + 4);
@@ -109,6 +130,8 @@ int muon_amd_validate_aol(const MuonAolDesc* descs, int nmat, const int32_t* row
         MUON_REQUIRE(d.m_p > 0 && d.n_p > 0 && d.m_p % 8 == 0 && d.n_p % 8 == 0 &&
                          d.m_p % AOL_ROWS_PER_BLOCK == 0 && d.n_p % AOL_ROWS_PER_BLOCK == 0,
                      "aol desc %d: padded sizes %d x %d", i, d.m_p, d.n_p);
+        MUON_REQUIRE(!d.rowsum || (d.m_p % 64 == 0 && d.ld_rowsum >= d.m_p / 64),
+                     "aol desc %d: row-sum slots %d for %d rows", i, d.ld_rowsum, d.m_p);
         MUON_REQUIRE(d.ld_n >= d.n_p && d.ld_m >= d.m_p && d.ld_n % 8 == 0 && d.ld_m % 8 == 0,
                      "aol desc %d: leading dimensions %d/%d for %d x %d", i, d.ld_n, d.ld_m, d.m_p, d.n_p);
         MUON_REQUIRE((reinterpret_cast<uintptr_t>(d.xr) % 16) == 0 && (reinterpret_cast<uintptr_t>(d.xc) % 16) == 0 &&
@@ -135,12 +158,23 @@ int muon_amd_aol_rowsum(const MuonAolDesc* descs_dev, const int32_t* row_prefix_
     return check_launch("aol_rowsum");
 }
 
+int muon_amd_aol_rowsum_finalize(const MuonAolDesc* descs_dev, const int32_t* row_prefix_dev, int nmat,
+                                 int nblocks, float eps, void* stream) {
+    MUON_REQUIRE(descs_dev && row_prefix_dev, "aol_rowsum_finalize: null table");
+    MUON_REQUIRE(nmat > 0 && nblocks > 0 && eps > 0.f, "aol_rowsum_finalize: nmat=%d nblocks=%d eps=%g", nmat, nblocks, eps);
+    hipLaunchKernelGGL(aol_rowsum_finalize_kernel, dim3(nblocks), dim3(AOL_THREADS), 0,
+                       static_cast<hipStream_t>(stream), descs_dev, row_prefix_dev, nmat, eps);
+    return check_launch("aol_rowsum_finalize");
+}
+
 int muon_amd_aol_rescale(const MuonAolDesc* descs_dev, const int32_t* seg_prefix_dev, int nmat,
-                         int nblocks, void* stream) {
+                         int nblocks, int mode, void* stream) {
     MUON_REQUIRE(descs_dev && seg_prefix_dev, "aol_rescale: null table");
     MUON_REQUIRE(nmat > 0 && nblocks > 0, "aol_rescale: nmat=%d nblocks=%d", nmat, nblocks);
+    MUON_REQUIRE(mode == MUON_AMD_AOL_SYMMETRIC || mode == MUON_AMD_AOL_ROWS_ONLY, "aol_rescale: mode=%d", mode);
     hipLaunchKernelGGL(aol_rescale_kernel, dim3(nblocks), dim3(AOL_THREADS), 0,
-                       static_cast<hipStream_t>(stream), descs_dev, seg_prefix_dev, nmat);
+                       static_cast<hipStream_t>(stream), descs_dev, seg_prefix_dev, nmat,
+                       mode == MUON_AMD_AOL_ROWS_ONLY ? 1 : 0);
     return check_launch("aol_rescale");
 }
 

@@ -239,7 +239,11 @@ constexpr int strip_stage_bytes(int WN) {
 // of CT (and C2T).  With APPLY, the orientation of the parameter goes through the fused parameter
 // step instead of a store, and the other orientation is not produced.  `stage` is this wave's
 // strip_stage_bytes(WN) of LDS.
-template <bool HAS_D, bool STREAM, bool APPLY, int WGN, int WM, int WN, int TM, int TN>
+// ROWSUM (a mirrored product without addend): per row of the result, the sum of |o| over the
+// wave's 64 columns goes to d.rowsum[row][col0 / 64]; for a mirrored tile the column sums over the
+// wave's WM rows go to the rows of the mirror image, d.rowsum[col][row0 / 64] (and zero to the other
+// slots of those WM rows), so that every slot of every row is written exactly once per launch.
+template <bool HAS_D, bool STREAM, bool APPLY, bool ROWSUM, int WGN, int WM, int WN, int TM, int TN>
 __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const u32x2 (&dv)[TM][TN][4],
                                                    const MuonGemmDesc& d, const MuonTileJob& job, float alpha,
                                                    float beta, float gamma, bool round_terms, char* stage,
@@ -268,9 +272,13 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
         id1[t] = static_cast<__bf16>(16 + rho == lr ? 1.0f : 0.0f);
     }
 
+    float colsum[TN];          // ROWSUM: |o| summed down this lane's 16 rows of every strip, per column tile
+#pragma unroll
+    for (int b = 0; b < TN; ++b) colsum[b] = 0.f;
 #pragma unroll
     for (int a = 0; a < TM; ++a) {
         uint32_t ot[TN][8];   // this strip's results moved back to accumulator layout, packed bf16 pairs
+        float rowpart = 0.f;  // ROWSUM: |o| summed along this lane's 32 of the strip's 64 columns
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
             f32x16 u;
@@ -308,6 +316,7 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
                     float t2 = HAS_D ? beta * dd[e] : 0.f;
                     if (round_terms) t2 = round_bf(t2);
                     o[4 * q + e] = round_bf(u[4 * q + e] + t2);
+                    if constexpr (ROWSUM) rowpart += fabsf(o[4 * q + e]);
                 }
                 if (do_d) {
                     u32x2 pk;
@@ -320,7 +329,17 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
                 const f32x16 w = tile_transpose_bf16(o, id0, id1);
 #pragma unroll
                 for (int k = 0; k < 8; ++k) ot[b][k] = pack2bf(w[2 * k], w[2 * k + 1]);
+                if constexpr (ROWSUM) {
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) colsum[b] += fabsf(w[k]);
+                }
             }
+        }
+        if constexpr (ROWSUM) {
+            // the partner lane (l ^ 32) owns the other 32 columns of the same row
+            const float total = rowpart + __shfl_xor(rowpart, 32, 64);
+            if (g == 0)
+                d.rowsum[static_cast<size_t>(row0 + a * 32 + lr) * d.ld_rowsum + col0 / 64] = total;
         }
         if (do_d) {
             // 16-byte chunks per row, whole rows per wave-wide store
@@ -371,6 +390,21 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
                     const size_t off = static_cast<size_t>(col0 + row) * d.ldct + row0 + a * 32 + ch * 8;
                     gstore16<STREAM>(d.CT + off, v);
                     if (d.C2T) gstore16<STREAM>(d.C2T + off, scale_bf16x8(v, gamma));
+                }
+            }
+        }
+    }
+    if constexpr (ROWSUM) {
+        if (do_t) {
+#pragma unroll
+            for (int b = 0; b < TN; ++b) {
+                // the partner lane owns the other 16 rows of every strip of the same column
+                const float total = colsum[b] + __shfl_xor(colsum[b], 32, 64);
+                if (g == 0) {
+                    float* const dst = d.rowsum + static_cast<size_t>(col0 + b * 32 + lr) * d.ld_rowsum + row0 / 64;
+                    dst[0] = total;
+#pragma unroll
+                    for (int z = 1; z < WM / 64; ++z) dst[z] = 0.f;
                 }
             }
         }
@@ -729,10 +763,11 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
                 ap.wd_factor = wd_factor;
                 ap.vec_ok = (ap.mat->cols % 8 == 0) && ((reinterpret_cast<uintptr_t>(ap.mat->param) & 15) == 0) &&
                             ((reinterpret_cast<uintptr_t>(ap.mat->out) & 15) == 0);
-                ns_epilogue_strips<true, Cfg::STREAM_STORES, true, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+                ns_epilogue_strips<true, Cfg::STREAM_STORES, true, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
             } else {
-                if (has_d) ns_epilogue_strips<true, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
-                else ns_epilogue_strips<false, Cfg::STREAM_STORES, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+                if (has_d) ns_epilogue_strips<true, Cfg::STREAM_STORES, false, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+                else if ((flags & MUON_AMD_GEMM_ROWSUM) && d.rowsum) ns_epilogue_strips<false, Cfg::STREAM_STORES, false, true, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
+                else ns_epilogue_strips<false, Cfg::STREAM_STORES, false, false, WGN, WM, WN, TM, TN>(acc, dv, d, job, alpha, beta, gamma, round_terms, stage, ap);
             }
         }
         if (!has_next) break;
@@ -951,6 +986,10 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJ
                          (reinterpret_cast<uintptr_t>(d.D) % 16) == 0,
                      "gemm desc %d: misaligned pointer", i);
         MUON_REQUIRE(!(d.C2 && !d.C) && !(d.C2T && !d.CT), "gemm desc %d: scaled copy needs its primary output", i);
+        MUON_REQUIRE(!d.rowsum || (d.C && d.CT == d.C && !d.D && d.colsn % 64 == 0 && d.ld_rowsum >= d.colsn / 64 &&
+                                   (reinterpret_cast<uintptr_t>(d.rowsum) % 4) == 0),
+                     "gemm desc %d: row sums need a mirrored product without addend and %d slots per row (ld_rowsum=%d)",
+                     i, d.colsn / 64, d.ld_rowsum);
     }
     for (int j = 0; j < njobs; ++j) {
         const MuonTileJob& t = jobs[j];

@@ -60,9 +60,12 @@ class _ChunkRuntime:
         self.chunk = chunk
         self.device = device
         gemm = chunk.gemm_descs(base)
-        for ph in range(5):
+        for ph in range(_plan.N_PHASES):
+            if ph == _plan.PH_POLY_FULL and chunk.poly_full_jobs is None:
+                continue
             jobs = (chunk.syrk_jobs if ph == _plan.PH_SYRK else
-                    chunk.sym_jobs if ph == _plan.PH_POLY else chunk.full_jobs)
+                    chunk.sym_jobs if ph == _plan.PH_POLY else
+                    chunk.poly_full_jobs if ph == _plan.PH_POLY_FULL else chunk.full_jobs)
             _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(gemm[ph]), chunk.nmat,
                                                   _lib.host_ptr(jobs), len(jobs), chunk.tile_class,
                                                   chunk.split_slots if ph == _plan.PH_SYRK else 0),
@@ -73,13 +76,15 @@ class _ChunkRuntime:
         parts = [gemm.reshape(-1).view(np.uint8), chunk.sym_jobs.view(np.uint8),
                  chunk.full_jobs.view(np.uint8), chunk.block_prefix.view(np.uint8),
                  chunk.tile_prefix.view(np.uint8), chunk.syrk_jobs.view(np.uint8)]
-        if chunk.variant == "aol4":
+        if chunk.aol:
             aol = chunk.aol_descs(base)
             _lib.check(lib.muon_amd_validate_aol(_lib.host_ptr(aol), chunk.nmat,
                                                  _lib.host_ptr(chunk.aol_row_prefix),
                                                  _lib.host_ptr(chunk.aol_seg_prefix)), "validate_aol")
             parts += [aol.view(np.uint8), chunk.aol_row_prefix.view(np.uint8),
                       chunk.aol_seg_prefix.view(np.uint8)]
+            if chunk.poly_full_jobs is not None:
+                parts.append(chunk.poly_full_jobs.view(np.uint8))
         offs, blob, cur = [], [], 0
         for p in parts:
             offs.append(cur)
@@ -90,7 +95,7 @@ class _ChunkRuntime:
             cur += len(p) + pad
         self.static = _upload(np.concatenate(blob), device)
         b = self.static.data_ptr()
-        self.gemm_ptr = [b + offs[0] + ph * chunk.nmat * _lib.GEMM_DESC.itemsize for ph in range(5)]
+        self.gemm_ptr = [b + offs[0] + ph * chunk.nmat * _lib.GEMM_DESC.itemsize for ph in range(_plan.N_PHASES)]
         self.sym_jobs_ptr = b + offs[1]
         self.full_jobs_ptr = b + offs[2]
         self.block_prefix_ptr = b + offs[3]
@@ -100,8 +105,9 @@ class _ChunkRuntime:
         self.split_counters = torch.zeros(max(chunk.split_slots, 1), dtype=torch.int32, device=device)
         self.split_partials_ptr = base + chunk.off_split_partials if chunk.split_slots else None
         self.split_counters_ptr = self.split_counters.data_ptr() if chunk.split_slots else None
-        if chunk.variant == "aol4":
+        if chunk.aol:
             self.aol_ptr, self.aol_row_prefix_ptr, self.aol_seg_prefix_ptr = (b + o for o in offs[6:9])
+            self.poly_full_jobs_ptr = b + offs[9] if chunk.poly_full_jobs is not None else None
         self.mat_dev = None
         self.mat_key = None
 
@@ -154,7 +160,7 @@ class _ChunkRuntime:
         _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
             int(mutate_grad), sc_mom, s), "momentum"))
-        norm_flags = flags | (_lib.NORM_UNIT if c.variant == "aol4" else 0)
+        norm_flags = flags | (_lib.NORM_UNIT if c.aol else 0)
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
             mats, c.nmat, eps, norm_flags, s), "norm_finalize"))
         _launch("normalize", elts * 2 + padded * 4, lambda: _lib.check(lib.muon_amd_normalize(
@@ -165,27 +171,37 @@ class _ChunkRuntime:
         }
         f_upd = sum(2 * lay.m * lay.m * lay.n for lay in c.layouts)
 
-        def gemm(name, ph, it, jobs_ptr, njobs, work):
+        def gemm(name, ph, it, jobs_ptr, njobs, work, extra_flags=0):
             al, be, ga = c.phase_scalars(ph, it)
             split = ph == _plan.PH_SYRK
             _launch(name, work, lambda: _lib.check(lib.muon_amd_ns_gemm(
-                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags,
+                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags | extra_flags,
                 self.split_partials_ptr if split else None, self.split_counters_ptr if split else None, s),
                 "ns_gemm"))
 
         for it in range(c.steps):
-            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.syrk_jobs_ptr, len(c.syrk_jobs), flops[_plan.PH_SYRK])
-            if c.variant == "aol4" and it == 0:
-                # muon.py:776-785: row sums of |A|, then X and A rescaled in place (A becomes the
-                # Gram matrix of the rescaled X, so this iteration needs no second X X^T)
+            first_aol = c.aol and it == 0
+            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.syrk_jobs_ptr, len(c.syrk_jobs), flops[_plan.PH_SYRK],
+                 _lib.GEMM_ROWSUM if first_aol else 0)
+            if first_aol:
+                # muon.py:776-785: the row sums of |A| come out of the product's epilogue as partial
+                # sums (one small launch adds them up), then X and A are rescaled in place (A becomes
+                # the Gram matrix of the rescaled X, so this iteration needs no second X X^T)
                 gram_bytes = sum(lay.mp * lay.mp * 2 for lay in c.layouts)
-                _launch("aol_rowsum", gram_bytes, lambda: _lib.check(lib.muon_amd_aol_rowsum(
+                part_bytes = sum(lay.mp * (lay.mp // _plan.ROWSUM_SLOT) * 4 for lay in c.layouts)
+                _launch("aol_rowsum_finalize", part_bytes, lambda: _lib.check(lib.muon_amd_aol_rowsum_finalize(
                     self.aol_ptr, self.aol_row_prefix_ptr, c.nmat, int(c.aol_row_prefix[-1]), eps, s),
-                    "aol_rowsum"))
+                    "aol_rowsum_finalize"))
+                mode = _lib.AOL_ROWS_ONLY if c.variant == "aol4_rows" else _lib.AOL_SYMMETRIC
                 _launch("aol_rescale", 2 * gram_bytes + 8 * padded, lambda: _lib.check(lib.muon_amd_aol_rescale(
-                    self.aol_ptr, self.aol_seg_prefix_ptr, c.nmat, int(c.aol_seg_prefix[-1]), s),
+                    self.aol_ptr, self.aol_seg_prefix_ptr, c.nmat, int(c.aol_seg_prefix[-1]), mode, s),
                     "aol_rescale"))
-            gemm("ns_gemm/poly", _plan.PH_POLY, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_POLY])
+            if first_aol and c.variant == "aol4_rows":
+                # A / s is not symmetric: c * A A^T + b * A over every tile, no mirrored store
+                gemm("ns_gemm/poly", _plan.PH_POLY_FULL, it, self.poly_full_jobs_ptr, len(c.poly_full_jobs),
+                     2 * flops[_plan.PH_POLY])
+            else:
+                gemm("ns_gemm/poly", _plan.PH_POLY, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_POLY])
             if it == c.steps - 1 and FOLD_APPLY:
                 # the last update product takes the parameter step in its epilogue (muon.py:14, 98-99)
                 al, be, _ = c.phase_scalars(_plan.PH_UPD_LAST, it)

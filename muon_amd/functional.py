@@ -79,18 +79,22 @@ def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float 
     return _orthogonalise(G, steps, epsilon, _rounding_flag(rounding), "ns5")
 
 
-def zeropower_via_aol4(G: torch.Tensor, epsilon: float = 1e-7) -> torch.Tensor:
+def zeropower_via_aol4(G: torch.Tensor, epsilon: float = 1e-7, *, rescale: str = "symmetric") -> torch.Tensor:
     """The 4-iteration variant with AOL rescaling (reference muon.py:748-799): instead of the
     Frobenius pre-scale, the rows of X are divided by sqrt(sum_j |(X X^T)_ij|), which bounds the
     spectral norm by 1 and starts closer to orthogonal; four quintic iterations with the
     coefficients of muon.py:754-759 follow, the first reusing the rescaled Gram matrix.
 
-    One deliberate difference: the Gram matrix is rescaled on both sides (it then is the Gram
-    matrix of the rescaled X); the reference divides its rows only (muon.py:785), which is not
-    symmetric, depends on its autotuned tile through its mirroring store, and loses the
-    contraction of the iteration for matrices with uneven row norms.
+    rescale="symmetric" (default) rescales the Gram matrix on both sides, diag(r) A diag(r): it
+    then is the Gram matrix of the rescaled X, which the iteration assumes.  rescale="rows" divides
+    its rows only, `A / s`, as muon.py:785 is written: A is then not symmetric, the first
+    polynomial c * A A^T + b * A is computed over every tile, and for matrices with uneven row
+    norms the iteration loses its contraction (the reference's own result further depends on the
+    tile its autotuner picked, through the mirrored store of its polynomial kernel).
     """
-    return _orthogonalise(G, len(AOL_COEFFS), epsilon, False, "aol4")
+    if rescale not in ("symmetric", "rows"):
+        raise ValueError(f"rescale must be 'symmetric' or 'rows', got {rescale!r}")
+    return _orthogonalise(G, len(AOL_COEFFS), epsilon, False, "aol4" if rescale == "symmetric" else "aol4_rows")
 
 
 def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,

@@ -27,8 +27,8 @@ class _MuonBase(torch.optim.Optimizer):
 
     def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5", use_graph=False):
         self._use_graph = bool(use_graph)
-        if ns_variant not in ("ns5", "aol4"):
-            raise ValueError(f"ns_variant must be 'ns5' or 'aol4', got {ns_variant!r}")
+        if ns_variant not in ("ns5", "aol4", "aol4_rows"):
+            raise ValueError(f"ns_variant must be 'ns5', 'aol4' or 'aol4_rows', got {ns_variant!r}")
         self._ns_variant = ns_variant
         self._ns_rounding = ns_rounding
         self._reference_rounding = _rounding_flag(ns_rounding)
@@ -214,7 +214,9 @@ class SingleDeviceMuon(_MuonBase):
     mutate_grad (write the Nesterov blend back into p.grad as the reference's in-place lerp does;
     off by default because nothing reads it), workspace_bytes (cap of the bf16 workspace),
     ns_variant ("ns5": the five-iteration specification muon.py:265-291; "aol4": the
-    four-iteration AOL-rescaled variant muon.py:748-799, see zeropower_via_aol4), use_graph
+    four-iteration AOL-rescaled variant muon.py:748-799 with the Gram matrix rescaled on both
+    sides, "aol4_rows": the same with `A / s` by rows only as muon.py:785 is written; see
+    zeropower_via_aol4), use_graph
     (record every launch of a step -- all Muon groups and all Adam groups on a device -- into one
     HIP graph once and replay it every step; tensor addresses and hyper-parameters are read from
     device memory, so gradients may be reallocated and learning rates scheduled between steps).

@@ -24,7 +24,8 @@ NS_COEFFS = (3.4445, -4.7750, 2.0315)   # reference muon.py:276
 # per-iteration coefficients of the 4-iteration AOL-rescaled variant, reference muon.py:754-759
 AOL_COEFFS = ((4.0098, -7.0585, 2.4635), (3.4585, -5.5479, 2.5959),
               (2.7573, -3.2939, 1.4254), (2.7215, -3.0494, 1.3169))
-VARIANTS = ("ns5", "aol4")
+# "aol4": the Gram matrix rescaled on both sides; "aol4_rows": by rows only, as muon.py:785 writes it
+VARIANTS = ("ns5", "aol4", "aol4_rows")
 AOL_ROWS = 4                            # must match muon_amd_aol_rows_per_block()
 TILE_DIMS = {0: (128, 128), 1: (256, 256)}   # must match muon_amd_gemm_tile_rows/cols()
 # output tiles (rows, cols) of one XCD-resident super-block: as many tiles as an XCD holds workgroups
@@ -39,7 +40,9 @@ N_XCD = 8                               # workgroups are dealt round-robin to th
 LD_PAD = int(os.environ.get("MUON_AMD_LD_PAD", "0"))
 _ALIGN = 256
 
-PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST = range(5)
+PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST, PH_POLY_FULL = range(6)
+N_PHASES = 6
+ROWSUM_SLOT = 64                        # columns per slot of the fused row sums (the wave tile's width)
 
 
 BIG_TILE_MIN_M = int(os.environ.get("MUON_AMD_BIG_TILE_MIN_M", "1024"))
@@ -158,7 +161,8 @@ class ChunkPlan:
     def __init__(self, mats, tile_class: int, steps: int, reference_rounding: bool, variant: str = "ns5"):
         # mats: list of (index, rows, cols)
         assert variant in VARIANTS
-        if variant == "aol4":           # fixed schedule, one rounding per stored matrix
+        self.aol = variant in ("aol4", "aol4_rows")
+        if self.aol:                    # fixed schedule, one rounding per stored matrix
             steps, reference_rounding = len(AOL_COEFFS), False
         self.variant = variant
         self.tile_class = tile_class
@@ -192,11 +196,14 @@ class ChunkPlan:
         off += _round_up(self.nblocks * 4, _ALIGN)
         self.off_denoms = off
         off += _round_up(self.nmat * 4, _ALIGN)
-        # AOL variant: r = s^-1/2 per row of each Gram matrix, and the block prefixes of its two launches
-        self.off_rvec = []
+        # AOL variants: r = s^-1/2 per row of each Gram matrix, the partial row sums the first X X^T
+        # launch leaves (one float per row and 64-column slot), and the block prefixes of the launches
+        self.off_rvec, self.off_rowsum = [], []
         for lay in self.layouts:
             self.off_rvec.append(off)
-            off += _round_up(lay.mp * 4, _ALIGN) if variant == "aol4" else 0
+            off += _round_up(lay.mp * 4, _ALIGN) if self.aol else 0
+            self.off_rowsum.append(off)
+            off += _round_up(lay.mp * (lay.mp // ROWSUM_SLOT) * 4, _ALIGN) if self.aol else 0
         rowblk = [lay.mp // AOL_ROWS for lay in self.layouts]
         self.aol_row_prefix = np.concatenate([[0], np.cumsum(rowblk)]).astype(np.int32)
         segblk = [b for lay in self.layouts for b in (lay.mp // AOL_ROWS, lay.np_ // AOL_ROWS, lay.mp // AOL_ROWS)]
@@ -207,6 +214,9 @@ class ChunkPlan:
         self.syrk_jobs = self._jobs(sym=True, reduce_over_n=True)
         self.sym_jobs = self._jobs(sym=True, reduce_over_n=False)
         self.full_jobs = self._jobs(sym=False, reduce_over_n=False)
+        # every tile of the m x m polynomial (no mirrored store): the first iteration of "aol4_rows",
+        # whose Gram matrix is not symmetric after the row-only rescaling
+        self.poly_full_jobs = self._jobs(sym=False, reduce_over_n=False, square=True) if variant == "aol4_rows" else None
         # fp32 slots of the split jobs (scratch like the rest; the per-slot counters are not part
         # of the workspace: they must stay zero between launches, and chunks share the workspace)
         self.off_split_partials = off
@@ -214,14 +224,14 @@ class ChunkPlan:
         self.workspace_bytes = off
 
     # ---- tile job lists -----------------------------------------------------------------
-    def _jobs(self, sym: bool, reduce_over_n: bool) -> np.ndarray:
+    def _jobs(self, sym: bool, reduce_over_n: bool, square: bool = False) -> np.ndarray:
         TR, TC = self.tile_rows, self.tile_cols
         ratio = TR // TC
         si, sj = SUPER_DIMS[self.tile_class]
         parts = []
         for k, lay in enumerate(self.layouts):
             mt = lay.mp // TR
-            nt = (lay.mp if sym else lay.np_) // TC
+            nt = (lay.mp if (sym or square) else lay.np_) // TC
             ti, tj = _tile_order(mt, nt, sym, ratio, si, sj)
             kdim = lay.np_ if reduce_over_n else lay.mp
             nsplit = split_factor(lay.mp, kdim) if reduce_over_n else 1
@@ -251,8 +261,8 @@ class ChunkPlan:
         return "X" if lay.wide else ("XT1" if self.steps % 2 else "XT0")
 
     def gemm_descs(self, base: int) -> np.ndarray:
-        """[5, nmat] MuonGemmDesc table for a workspace at device address `base`."""
-        d = np.zeros((5, self.nmat), dtype=_lib.GEMM_DESC)
+        """[N_PHASES, nmat] MuonGemmDesc table for a workspace at device address `base`."""
+        d = np.zeros((N_PHASES, self.nmat), dtype=_lib.GEMM_DESC)
         for k, lay in enumerate(self.layouts):
             p = {name: base + o for name, o in lay.off.items()}
             mp, np_ = lay.mp, lay.np_
@@ -265,6 +275,9 @@ class ChunkPlan:
                 s["C2"] = s["C2T"] = p["CA"]
             s["ldc"] = s["ldct"] = lay.ldm
             s["rows"] = s["colsn"] = mp
+            if self.aol:                # used by the launch that carries MUON_AMD_GEMM_ROWSUM only
+                s["rowsum"] = base + self.off_rowsum[k]
+                s["ld_rowsum"] = mp // ROWSUM_SLOT
             q = d[PH_POLY, k]
             q["P"] = p["CA"] if self.reference_rounding else p["A"]
             q["Q"] = q["D"] = p["A"]
@@ -273,6 +286,10 @@ class ChunkPlan:
             q["C"] = q["CT"] = p["B"]
             q["ldc"] = q["ldct"] = lay.ldm
             q["rows"] = q["colsn"] = mp
+            f = d[PH_POLY_FULL, k]      # the polynomial over every tile, stored in one orientation
+            for name in _lib.GEMM_DESC.names:
+                f[name] = q[name]
+            f["CT"] = 0
             for ph, src, dst in ((PH_UPD_EVEN, "XT0", "XT1"), (PH_UPD_ODD, "XT1", "XT0")):
                 u = d[ph, k]
                 u["P"] = p["B"]
@@ -330,15 +347,17 @@ class ChunkPlan:
             r["xc"] = base + lay.off["XT0"]
             r["gram"] = base + lay.off["A"]
             r["rvec"] = base + self.off_rvec[k]
+            r["rowsum"] = base + self.off_rowsum[k]
+            r["ld_rowsum"] = lay.mp // ROWSUM_SLOT
             r["m_p"], r["n_p"], r["ld_n"], r["ld_m"] = lay.mp, lay.np_, lay.ldn, lay.ldm
         return d
 
     def phase_scalars(self, phase: int, iteration: int = 0):
         """(alpha, beta, gamma) of the GEMM epilogue for a phase of an iteration."""
-        a, b, c = AOL_COEFFS[iteration] if self.variant == "aol4" else NS_COEFFS
+        a, b, c = AOL_COEFFS[iteration] if self.aol else NS_COEFFS
         if phase == PH_SYRK:
             return 1.0, 0.0, c
-        if phase == PH_POLY:
+        if phase in (PH_POLY, PH_POLY_FULL):
             return (1.0, b, 0.0) if self.reference_rounding else (c, b, 0.0)
         return 1.0, a, 0.0
 

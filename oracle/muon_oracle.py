@@ -13,6 +13,7 @@ implementation (all citations are into /root/reference/muon.py):
   ns_aol4                    muon.py:748-799  (the live 4-iteration variant with AOL rescaling,
                              built on the Triton kernels muon.py:349-746; see its docstring
                              for what of it can and cannot be pinned)
+  ns_aol4_rows               the same with muon.py:785 (`A / s`, rows only) taken as written
   muon_update                muon.py:8-15
   adam_update                muon.py:104-109
   OracleSingleDeviceMuon     muon.py:73-101
@@ -45,6 +46,12 @@ What pins each function (the reference ships no tests, golden vectors or fixture
                      quintics applied to its singular values), by orthogonal and diagonal
                      inputs (both reduce to the scalar chain at 1), the AOL bound
                      sigma_max(diag(r) X) <= 1, the transpose rule and batched == per-matrix.
+  * ns_aol4_rows  -- the literal reading of muon.py:785.  Pinned by a python-loop float64
+                     restatement on tiny matrices, by inputs whose row sums s_i are all equal
+                     (then it is ns_aol4: orthogonal and scaled-orthogonal inputs), and by the
+                     diagonal case.  PARITY UNPINNED against the reference's live code for the
+                     same reasons as ns_aol4; in addition the reference's mirrored store makes
+                     its own output depend on the autotuned block size, which is not restated.
 No other function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -112,6 +119,60 @@ def ns_aol4(G: torch.Tensor, epsilon: float = 1e-7, work_dtype: torch.dtype = to
         X = (a * X.to(acc) + B.to(acc) @ X.to(acc)).to(work_dtype)                    # ns_line_3, muon.py:787, 794
     if tall:                                                       # muon.py:797-798
         X = X.mT
+    return X
+
+
+def ns_aol4_rows(G: torch.Tensor, epsilon: float = 1e-7, work_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """muon.py:748-799 with `A = A / s` taken as written (muon.py:785: the rows of the Gram matrix
+    are divided, its columns are not), at the level of the tensor expressions and of what the
+    docstrings of the three kernels state (ns_line_1: X X^T, muon.py:364; ns_line_2:
+    alpha A A^T + beta A, muon.py:485; ns_line_3: a X + B X).  The reference's polynomial kernel
+    stores every block it computes and its transpose (muon.py:538-552), so on this non-symmetric A
+    its own result depends on the block size its autotuner picked; that artefact is not restated
+    here: B is the full, unmirrored alpha A A^T + beta A.  Roundings as in ns_aol4."""
+    assert G.ndim >= 2
+    acc = torch.float64 if work_dtype == torch.float64 else torch.float32
+    X = G.to(work_dtype)
+    tall = G.size(-2) > G.size(-1)
+    if tall:
+        X = X.mT
+    gram = lambda Y: _upper_mirrored((Y.to(acc) @ Y.to(acc).mT).to(work_dtype))
+    A = gram(X)                                                    # muon.py:778
+    s = torch.clamp_min(A.to(acc).abs().sum(dim=-1, keepdim=True).to(work_dtype).to(acc), epsilon)  # muon.py:779-781
+    r = torch.rsqrt(s)
+    X = (X.to(acc) * r).to(work_dtype)                             # muon.py:782
+    A = (A.to(acc) * (r * r)).to(work_dtype)                       # muon.py:785: A / s, rows only
+    for it, (a, b, c) in enumerate(AOL_CONSTS):
+        if it > 0:
+            A = gram(X)
+        Af = A.to(acc)
+        F = (c * (Af @ Af.mT) + b * Af).to(work_dtype)             # ns_line_2
+        B = F if it == 0 else _upper_mirrored(F)                   # symmetric from the second iteration on
+        X = (a * X.to(acc) + B.to(acc) @ X.to(acc)).to(work_dtype)
+    if tall:
+        X = X.mT
+    return X
+
+
+def ns_aol4_rows_brute_force(G_rows, epsilon: float = 1e-7):
+    """ns_aol4_rows in float64 with python loops only (lists of lists; wide or square input): an
+    independent restatement for tiny matrices."""
+    X = [[float(v) for v in row] for row in G_rows]
+    m, n = len(X), len(X[0])
+    assert m <= n
+    mm = lambda P, Q: [[sum(P[i][k] * Q[k][j] for k in range(len(Q))) for j in range(len(Q[0]))] for i in range(len(P))]
+    tr = lambda P: [list(col) for col in zip(*P)]
+    A = mm(X, tr(X))
+    s = [max(sum(abs(v) for v in row), epsilon) for row in A]
+    X = [[X[i][j] / s[i] ** 0.5 for j in range(n)] for i in range(m)]
+    A = [[A[i][j] / s[i] for j in range(m)] for i in range(m)]
+    for it, (a, b, c) in enumerate(AOL_CONSTS):
+        if it > 0:
+            A = mm(X, tr(X))
+        AAt = mm(A, tr(A))
+        B = [[c * AAt[i][j] + b * A[i][j] for j in range(m)] for i in range(m)]
+        BX = mm(B, X)
+        X = [[a * X[i][j] + BX[i][j] for j in range(n)] for i in range(m)]
     return X
 
 

@@ -537,6 +537,38 @@ def test_aol4_matches_oracle_and_closed_form(M, shape, std):
     assert O.rel_fro(got.double(), O.ns_aol4_closed_form(G.bfloat16().double().numpy())) <= TOL_FP32
 
 
+@pytest.mark.parametrize("shape,std", [((768, 3072), 1e-3), ((3072, 768), 1e-3), ((1024, 2048), 1e-4), ((64, 216), 1e-2),
+                                       ((130, 300), 1.0), ((128, 8192), 1e-2)])
+def test_aol4_rows_only_rescaling_matches_its_oracle(M, shape, std):
+    """rescale="rows" (muon.py:785 as written: A / s by rows, the first polynomial over every tile)
+    against the oracle's restatement in bf16 and float64, on matrices whose row norms vary by
+    +-10 % (with strongly uneven rows this map is not a contraction and nothing can be compared)."""
+    torch.manual_seed(hash(shape) % 1000 + 1)
+    G = torch.randn(*shape) * std * (1 + 0.2 * (torch.rand(shape[0], 1) - 0.5))
+    got = M.zeropower_via_aol4(_dev(G), rescale="rows")
+    assert got.dtype == torch.bfloat16 and got.shape == G.shape
+    got = got.float().cpu()
+    assert O.rel_fro(got, O.ns_aol4_rows(G).float()) <= TOL_BF16
+    assert O.rel_fro(got.double(), O.ns_aol4_rows(G.bfloat16().double(), work_dtype=torch.float64)) <= TOL_FP32
+    sym = M.zeropower_via_aol4(_dev(G)).float().cpu()
+    assert O.rel_fro(sym, O.ns_aol4(G).float()) <= TOL_BF16      # the default is still the two-sided rescaling
+    with pytest.raises(ValueError):
+        M.zeropower_via_aol4(_dev(G), rescale="columns")
+
+
+def test_aol4_rows_only_optimizer_step(M):
+    shapes = [(256, 384), (384, 256), (16, 8, 3, 3)]
+    cpu, gpu = _clone_params(shapes, 0.02, 1322)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns=O.ns_aol4_rows)
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns_variant="aol4_rows")
+    for step in range(2):
+        _set_grads(cpu, gpu, 1e-2)
+        oc.step()
+        og.step()
+        for pc, pg in zip(cpu, gpu):
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 2e-3, (tuple(pc.shape), step)
+
+
 def test_aol4_batched_special_inputs_and_optimizer_step(M):
     torch.manual_seed(1320)
     Gb = torch.randn(5, 96, 160) * 1e-2

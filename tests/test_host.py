@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     lib = _lib.load()
-    assert lib.muon_amd_abi_version() == 1
+    assert lib.muon_amd_abi_version() == 2
     for tc, (tr, tcol) in plan.TILE_DIMS.items():
         assert (lib.muon_amd_gemm_tile_rows(tc), lib.muon_amd_gemm_tile_cols(tc)) == (tr, tcol)
     assert lib.muon_amd_gemm_tile_rows(7) < 0 and b"tile class" in lib.muon_amd_last_error()
@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_the_library():
     lib = _lib.load()
     assert _lib.MAT_DESC.itemsize == lib.muon_amd_sizeof_mat_desc() == 120
-    assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 88
+    assert _lib.GEMM_DESC.itemsize == lib.muon_amd_sizeof_gemm_desc() == 104
     assert _lib.TILE_JOB.itemsize == lib.muon_amd_sizeof_tile_job() == 32
     assert _lib.ADAM_DESC.itemsize == lib.muon_amd_sizeof_adam_desc() == 56
 
@@ -282,21 +282,43 @@ def test_aol_variant_plan_validates():
     in the workspace, and block prefixes the library accepts."""
     lib = _lib.load()
     assert lib.muon_amd_aol_rows_per_block() == plan.AOL_ROWS
-    assert _lib.AOL_DESC.itemsize == lib.muon_amd_sizeof_aol_desc() == 48
+    assert _lib.AOL_DESC.itemsize == lib.muon_amd_sizeof_aol_desc() == 64
+    for variant in ("aol4", "aol4_rows"):
+        chunks = plan.plan_chunks(SHAPES, 5, True, 1 << 30, variant)
+        for c in chunks:
+            assert c.variant == variant and c.aol and c.steps == len(plan.AOL_COEFFS) == 4 and not c.reference_rounding
+            d = c.aol_descs(1 << 20)
+            rc = lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix),
+                                           _lib.host_ptr(c.aol_seg_prefix))
+            assert rc == 0, lib.muon_amd_last_error()
+            assert [c.phase_scalars(plan.PH_POLY, it) for it in range(4)] == [(co[2], co[1], 0.0) for co in plan.AOL_COEFFS]
+            assert c.phase_scalars(plan.PH_UPD_EVEN, 2) == (1.0, plan.AOL_COEFFS[2][0], 0.0)
+            g = c.gemm_descs(1 << 20)
+            for k, l in enumerate(c.layouts):
+                # the r vectors and the partial row sums lie inside the workspace, apart from everything else
+                assert c.off_denoms + 4 * c.nmat <= c.off_rvec[k] and c.off_rvec[k] + 4 * l.mp <= c.off_rowsum[k]
+                assert c.off_rowsum[k] + 4 * l.mp * (l.mp // 64) <= c.workspace_bytes
+                assert g[plan.PH_SYRK, k]["rowsum"] == (1 << 20) + c.off_rowsum[k] == d[k]["rowsum"]
+                assert g[plan.PH_SYRK, k]["ld_rowsum"] == l.mp // 64 == d[k]["ld_rowsum"]
+            rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[plan.PH_SYRK]), c.nmat, _lib.host_ptr(c.syrk_jobs),
+                                            len(c.syrk_jobs), c.tile_class, c.split_slots)
+            assert rc == 0, lib.muon_amd_last_error()
+            if variant == "aol4_rows":      # every tile of the m x m polynomial once, stored in one orientation
+                TR, TC = c.tile_rows, c.tile_cols
+                rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[plan.PH_POLY_FULL]), c.nmat, _lib.host_ptr(c.poly_full_jobs),
+                                                len(c.poly_full_jobs), c.tile_class, 0)
+                assert rc == 0, lib.muon_amd_last_error()
+                assert g[plan.PH_POLY_FULL, 0]["CT"] == 0 and g[plan.PH_POLY_FULL, 0]["C"] == g[plan.PH_POLY, 0]["C"]
+                for k, l in enumerate(c.layouts):
+                    pj = c.poly_full_jobs[c.poly_full_jobs["desc"] == k]
+                    got = sorted(zip((pj["i0"] // TR).tolist(), (pj["j0"] // TC).tolist()))
+                    assert got == [(i, j) for i in range(l.mp // TR) for j in range(l.mp // TC)]
+            else:
+                assert c.poly_full_jobs is None
+            bad = c.aol_seg_prefix.copy()
+            bad[1] += 1
+            assert lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix), _lib.host_ptr(bad)) == -1
     chunks = plan.plan_chunks(SHAPES, 5, True, 1 << 30, "aol4")
-    for c in chunks:
-        assert c.variant == "aol4" and c.steps == len(plan.AOL_COEFFS) == 4 and not c.reference_rounding
-        d = c.aol_descs(1 << 20)
-        rc = lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix),
-                                       _lib.host_ptr(c.aol_seg_prefix))
-        assert rc == 0, lib.muon_amd_last_error()
-        assert [c.phase_scalars(plan.PH_POLY, it) for it in range(4)] == [(co[2], co[1], 0.0) for co in plan.AOL_COEFFS]
-        assert c.phase_scalars(plan.PH_UPD_EVEN, 2) == (1.0, plan.AOL_COEFFS[2][0], 0.0)
-        for k, l in enumerate(c.layouts):      # the r vectors lie inside the workspace, apart from everything else
-            assert c.off_denoms + 4 * c.nmat <= c.off_rvec[k] and c.off_rvec[k] + 4 * l.mp <= c.workspace_bytes
-        bad = c.aol_seg_prefix.copy()
-        bad[1] += 1
-        assert lib.muon_amd_validate_aol(_lib.host_ptr(d), c.nmat, _lib.host_ptr(c.aol_row_prefix), _lib.host_ptr(bad)) == -1
     ns5 = plan.plan_chunks(SHAPES, 5, True, 1 << 30)
     assert all(a.workspace_bytes > b.workspace_bytes for a, b in zip(chunks, ns5))
 

@@ -321,6 +321,30 @@ def test_row_only_rescaling_of_the_gram_matrix_is_not_a_contraction():
     assert torch.linalg.svdvals(O.ns_aol4(G, work_dtype=torch.float64)).max() < 1.25
 
 
+def test_aol4_rows_only_restatement():
+    """ns_aol4_rows (muon.py:785 as written: the rows of the Gram matrix divided, its columns not):
+    against a python-loop float64 restatement on tiny matrices with mildly uneven rows, where it
+    differs from the two-sided rescaling; equal to it when every row sum s_i is the same."""
+    for seed in range(4):
+        g = torch.Generator().manual_seed(seed)
+        Q, _ = torch.linalg.qr(torch.randn(8, 5, dtype=torch.float64, generator=g))
+        scale = torch.tensor([1.0, 1.1, 0.9, 1.05, 0.95], dtype=torch.float64)[:, None]
+        G = (Q.mT + 0.05 * torch.randn(5, 8, dtype=torch.float64, generator=g)) * scale
+        got = O.ns_aol4_rows(G, work_dtype=torch.float64)
+        want = torch.tensor(O.ns_aol4_rows_brute_force(G.tolist()), dtype=torch.float64)
+        assert (got - want).abs().max() < 1e-12
+        assert (got - O.ns_aol4(G, work_dtype=torch.float64)).abs().max() > 1e-2       # not the same map
+        tall = O.ns_aol4_rows(G.mT.contiguous(), work_dtype=torch.float64)             # transpose rule, muon.py:761-762, 797-798
+        assert (tall.mT - got).abs().max() < 1e-12
+    Q, _ = torch.linalg.qr(torch.randn(24, 24, dtype=torch.float64, generator=torch.Generator().manual_seed(9)))
+    for G in (Q, 3.0 * Q, torch.diag(torch.tensor([0.5, -2.0, 3.0], dtype=torch.float64))):
+        # equal row sums (orthogonal input), and a diagonal input (A and A / s are diagonal: symmetric)
+        assert (O.ns_aol4_rows(G, work_dtype=torch.float64) - O.ns_aol4(G, work_dtype=torch.float64)).abs().max() < 1e-12
+    G = torch.randn(64, 96, generator=torch.Generator().manual_seed(10))
+    assert O.rel_fro(O.ns_aol4_rows(G).float(), O.ns_aol4_rows(G.double(), work_dtype=torch.float64)) < 2e-2   # bf16 storage
+    assert torch.count_nonzero(O.ns_aol4_rows(torch.zeros(8, 12))) == 0
+
+
 def test_aol4_golden_fixture_is_what_the_oracle_computes(golden_dir):
     z = np.load(os.path.join(golden_dir, "aol4_golden.npz"))
     for name in sorted({k.split("/")[0] for k in z.files}):
