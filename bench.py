@@ -92,13 +92,29 @@ def correctness_gates(name):
         if not value <= bound:
             failed.append(f"{key} = {value:.3e} > {bound:.3e}")
 
+    def ns_gates(tag, g2):
+        """Newton-Schulz output for the 2-D input g2 (CPU tensor).  The oracle's bf16 tensor
+        expressions are evaluated twice: by torch on the CPU, and by torch on this GPU (bf16
+        torch.matmul = rocBLAS, the library the reference itself multiplies with).  Both accumulate
+        in fp32 but in different orders, and on strongly rectangular matrices (4096 x 14336) the
+        iteration amplifies that to more than 2e-2 between the two evaluations of the SAME
+        expressions; the bound on the distance to the CPU evaluation is therefore the larger of 2e-2
+        and the distance between the two evaluations (+5e-3).  The distance to the GPU evaluation
+        is held to 2e-2 everywhere."""
+        got = muon_amd.zeropower_via_newtonschulz5(g2.cuda()).float().cpu()
+        ref16, ref32 = O.ns5_bf16(g2).float(), O.ns5_fp32(g2.float())
+        ref16_gpu = O.ns5_bf16(g2.cuda()).float().cpu()
+        spread = O.rel_fro(ref16_gpu, ref16)
+        res[f"ns_bf16_oracle_cpu_vs_gpu_evaluation_{tag}"] = round(float(spread), 6)
+        gate(f"ns_vs_bf16_gpu_evaluated_{tag}", O.rel_fro(got, ref16_gpu), TOL_NS_BF16)
+        gate(f"ns_vs_bf16_{tag}", O.rel_fro(got, ref16), max(TOL_NS_BF16, spread + 5e-3))
+        # where the reference's own bf16 result is further than 3e-2 from fp32 (small conv
+        # shapes), the kernel that follows its rounding sequence inherits that distance
+        gate(f"ns_vs_fp32_{tag}", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+
     torch.manual_seed(97)
     if name == "ns32":
-        G = torch.randn(4096, 4096).bfloat16()
-        got = muon_amd.zeropower_via_newtonschulz5(G.cuda()).float().cpu()
-        ref16, ref32 = O.ns5_bf16(G).float(), O.ns5_fp32(G.float())
-        gate("ns_vs_bf16_4096x4096", O.rel_fro(got, ref16), TOL_NS_BF16)
-        gate("ns_vs_fp32_4096x4096", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+        ns_gates("4096x4096", torch.randn(4096, 4096).bfloat16())
     else:
         muon, adam, gstd, _, _ = workload_shapes(name)
         for shape, _ in muon:
@@ -107,13 +123,7 @@ def correctness_gates(name):
             p_g = torch.nn.Parameter(p_c.detach().clone().cuda())
             g = torch.randn(*shape) * gstd
             p_c.grad, p_g.grad = g.clone(), g.clone().cuda()
-            g2 = g.reshape(mat2d(shape))
-            got = muon_amd.zeropower_via_newtonschulz5(g2.cuda()).float().cpu()
-            ref16, ref32 = O.ns5_bf16(g2).float(), O.ns5_fp32(g2)
-            gate(f"ns_vs_bf16_{tag}", O.rel_fro(got, ref16), TOL_NS_BF16)
-            # where the reference's own bf16 result is further than 3e-2 from fp32 (small conv
-            # shapes), the kernel that follows its rounding sequence inherits that distance
-            gate(f"ns_vs_fp32_{tag}", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+            ns_gates(tag, g.reshape(mat2d(shape)))
             O.OracleSingleDeviceMuon([p_c], lr=0.02, weight_decay=0.01, momentum=0.95).step()
             muon_amd.SingleDeviceMuon([p_g], lr=0.02, weight_decay=0.01, momentum=0.95).step()
             # a tiny filter's update is several per cent of |p|, so bf16 Newton-Schulz noise weighs more there
@@ -295,6 +305,8 @@ def secondary(name, gates):
         _, _, _, dsteps, dwarm = workload_shapes(name)
         r = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name])
     _, gw, gms, gn = summarize_kernels(r["per_label"])
+    if name != "ns32":
+        out["torch_gpu_baseline_ms_per_step"] = torch_gpu_baseline(name, steps=3)["ms_per_step"]
     out.update({"ms_per_step": round(r["ms_per_step"], 3), "ns_tflops_sym": round(gw / gms / 1e9, 1),
                 "ns_frac_of_peak": round(gw / gms / 1e9 / PEAK_BF16_TFLOPS, 4), "gemm_launches": gn,
                 "avg_gemm_launch_ms": round(gms / gn, 4)})
@@ -302,6 +314,72 @@ def secondary(name, gates):
         g = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], use_graph=True)
         out["ms_per_step_graph_replay"] = round(g["ms_per_step"], 3)
     return out
+
+
+# ------------------------------------------------------------------------------------------
+# Library baseline on the same GPU: the reference's step written with torch operations (bf16
+# torch.matmul = rocBLAS / hipBLASLt for the Newton-Schulz products, one parameter after the other,
+# nothing fused) -- what the reference's algorithm costs on this GPU without this library.
+# ------------------------------------------------------------------------------------------
+def torch_gpu_baseline(name, steps=2, warmup=1):
+    muon, adam, gstd, _, _ = workload_shapes(name)
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(77)
+    a, b, c = 3.4445, -4.7750, 2.0315                          # muon.py:276
+    lr, wd, beta = 0.02, 0.01, 0.95
+
+    def ns5(G):                                                # muon.py:265-291
+        X = G.bfloat16()
+        tall = G.size(-2) > G.size(-1)
+        if tall:
+            X = X.mT
+        X = X / (X.norm(dim=(-2, -1), keepdim=True) + 1e-7)
+        for _ in range(5):
+            A = X @ X.mT
+            B = b * A + c * A @ A
+            X = a * X + B @ X
+        return X.mT if tall else X
+
+    pm = [torch.randn(*shape, device=dev, generator=gen) * 0.02 for shape, count in muon for _ in range(count)]
+    pa = [torch.randn(*shape, device=dev, generator=gen) * 0.02 for shape, count in adam for _ in range(count)]
+    gm = [torch.randn_like(p) * gstd for p in pm]
+    ga = [torch.randn_like(p) * gstd for p in pa]
+    mom = [torch.zeros_like(p) for p in pm]
+    ea, eas = [torch.zeros_like(p) for p in pa], [torch.zeros_like(p) for p in pa]
+
+    def step(t):
+        for p, g0, m in zip(pm, gm, mom):                      # muon.py:8-15, 97-99
+            g = g0.clone()                                     # the reference overwrites p.grad; keep ours for the next step
+            m.lerp_(g, 1 - beta)
+            u = g.lerp_(m, beta)
+            if u.ndim == 4:
+                u = u.view(len(u), -1)
+            u = ns5(u)
+            u *= max(1, g.size(-2) / g.size(-1)) ** 0.5
+            p.mul_(1 - lr * wd)
+            p.add_(u.reshape(p.shape), alpha=-lr)
+        for p, g, m, v in zip(pa, ga, ea, eas):                # muon.py:104-109, 257-258
+            m.lerp_(g, 0.1)
+            v.lerp_(g.square(), 0.05)
+            upd = (m / (1 - 0.9 ** t)) / ((v / (1 - 0.95 ** t)).sqrt() + 1e-10)
+            p.mul_(1 - 3e-4 * wd)
+            p.add_(upd, alpha=-3e-4)
+
+    with torch.no_grad():
+        for t in range(1, warmup + 1):
+            step(t)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for t in range(warmup + 1, warmup + steps + 1):
+            step(t)
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    del pm, pa, gm, ga, mom, ea, eas
+    torch.cuda.empty_cache()
+    return dict(ms_per_step=round(ms, 3), steps=steps,
+                what="the reference step (muon.py:8-15, 97-109, 257-258, 265-291) as torch operations on this GPU: "
+                     "bf16 torch.matmul for the Newton-Schulz products, per parameter, unfused")
 
 
 # ------------------------------------------------------------------------------------------
@@ -394,6 +472,8 @@ def main():
                          "set_to_none=True) does), so that re-binding the descriptor tables is timed")
     ap.add_argument("--no-gates", action="store_true", help="skip the correctness gates (profiling runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-torch-baseline", action="store_true",
+                    help="skip timing the same step written with torch operations on this GPU")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations (GPT-2, ns32, conv)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first run one plain 1 GiB device-to-device copy kernel (a known-size reference "
@@ -484,6 +564,9 @@ def main():
         line["gpt2_124m"] = secondary("gpt2-124m", not args.no_gates)
         line["ns32"] = secondary("ns32", not args.no_gates)
         line["conv"] = secondary("conv", not args.no_gates)
+    if not args.no_torch_baseline:
+        line["torch_gpu_baseline"] = torch_gpu_baseline(args.workload)
+        line["torch_gpu_baseline"]["speedup"] = round(line["torch_gpu_baseline"]["ms_per_step"] / res["ms_per_step"], 2)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.workload)
         if line["cpu_baseline"]["value"]:
