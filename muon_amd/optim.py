@@ -2,8 +2,9 @@
 assertions (reference muon.py:18-70, 73-101, 112-199, 202-260), single-GPU semantics.
 
 Each `step()` issues, per Muon parameter group, a handful of grouped launches over all matrices
-of the group (momentum -> norm -> normalise -> 15 Newton-Schulz GEMM launches -> apply) and one
-fused launch per Adam group; nothing in it synchronises with the host.
+of the group (momentum -> norm -> normalise -> 15 Newton-Schulz GEMM launches, the last of which
+applies the update to the parameters) and one fused launch per Adam group; nothing in it
+synchronises with the host.
 """
 from __future__ import annotations
 
