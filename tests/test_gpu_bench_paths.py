@@ -178,3 +178,36 @@ def test_embedding_sized_adam_tensor_slabs(M):
                                            rtol=TOL_ADAM, atol=1e-16)
         np.testing.assert_allclose(v.detach().cpu().numpy(), cpu_v.detach().numpy(), rtol=TOL_ADAM, atol=1e-9)
         del g
+
+
+def test_workgroups_that_walk_several_jobs_keep_every_path_right(M):
+    """A launch never has more workgroups than the GPU holds at once (512 of the 128 x 128 class), so
+    with more jobs than that a workgroup computes several, fetching the next one's operands while it
+    writes the current one's results.  Batches large enough for that, on the paths that differ from
+    the plain one: split reductions (a job that only parks its partial sums goes straight on to its
+    next job), the fused row sums of the AOL variant, and the fused parameter step; each equal, bit
+    for bit, to the one-matrix run (whose launches have one job per workgroup), and one matrix per
+    batch against the oracle."""
+    torch.manual_seed(1430)
+    wide = torch.randn(80, 128, 8192) * 1e-2                    # 80 tiles x 8 split jobs = 640 jobs
+    got = M.zeropower_via_newtonschulz5(wide.cuda())
+    for b in (0, 41, 79):
+        assert torch.equal(M.zeropower_via_newtonschulz5(wide[b].cuda()), got[b]), b
+    assert O.rel_fro(got[79].float().cpu(), O.ns5_bf16(wide[79]).float()) <= TOL_BF16
+    sq = torch.randn(30, 768, 768) * 1e-3                       # 30 x 21 = 630 symmetric jobs, 30 x 36 update jobs
+    for fn, oracle in ((M.zeropower_via_aol4, O.ns_aol4), (M.zeropower_via_newtonschulz5, O.ns5_bf16)):
+        got = fn(sq.cuda())
+        for b in (0, 17, 29):
+            assert torch.equal(fn(sq[b].cuda()), got[b]), (fn.__name__, b)
+        assert O.rel_fro(got[29].float().cpu(), oracle(sq[29]).float()) <= TOL_BF16, fn.__name__
+    M.clear_engine_cache()
+    # fused parameter step over 24 x 36 = 864 jobs, tall and wide, against the oracle
+    shapes = [(768, 768)] * 12 + [(768, 1536)] * 4 + [(1536, 768)] * 4
+    cpu, gpu = _pair(shapes, 0.02, 1431)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95)
+    _grads(cpu, [gpu], 1e-3)
+    oc.step()
+    og.step()
+    for pc, pg in zip(cpu, gpu):
+        assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= TOL_PARAM, tuple(pc.shape)
