@@ -224,6 +224,70 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_grap
                 f_sym=fs, f_dense=fd)
 
 
+def run_backward_overlap(name, iters=10, warmup=3, tokens=65536, seed=4321):
+    """A training iteration = zero_grad, a synthetic backward, step(), with and without
+    overlap_backward.  The backward is what autograd does for the weights of linear layers fed a
+    batch of `tokens` tokens under bf16 autocast: one weight-gradient product x^T . dy per Muon
+    matrix (for a conv filter, of its flattened form), an elementwise gradient for the Adam tensors.
+    Reported per mode: the whole iteration and the step() call alone (HIP events on the launch
+    stream; the work the hooks move out of step() runs inside the iteration either way)."""
+    import muon_amd
+
+    muon, adam, _, _, _ = workload_shapes(name)
+    dev = torch.device("cuda:0")
+    out = {"backward": f"synthetic: weight-gradient products of a {tokens}-token batch, bf16 autocast", "iters": iters}
+    for mode in ("off", "on"):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(seed)
+        pm = [torch.nn.Parameter(torch.randn(*shape, device=dev, generator=gen) * 0.02)
+              for shape, count in muon for _ in range(count)]
+        pa = [torch.nn.Parameter(torch.randn(*shape, device=dev, generator=gen) * 0.02)
+              for shape, count in adam for _ in range(count)]
+        xs, dys, by_width = [], [], {}
+        for p in pm:                              # one input / output gradient per width, shared
+            r, c = mat2d(tuple(p.shape))
+            for w in (r, c):
+                if w not in by_width:
+                    by_width[w] = (torch.randn(tokens, w, device=dev, generator=gen) * 1e-2).bfloat16()
+            xs.append(by_width[r])
+            dys.append(by_width[c])
+        coef = [torch.randn_like(p) * 1e-3 for p in pa]
+        opt = muon_amd.SingleDeviceMuonWithAuxAdam([
+            dict(params=pm, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01),
+            dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)],
+            overlap_backward=(mode == "on"))
+
+        def iteration(ev=None):
+            opt.zero_grad(set_to_none=True)
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                loss = sum(((x @ p.reshape(x.shape[1], -1)) * dy).sum() for p, x, dy in zip(pm, xs, dys))
+            loss = loss + sum((p * c).sum() for p, c in zip(pa, coef))
+            loss.backward()
+            if ev is not None:
+                ev[0].record()
+            opt.step()
+            if ev is not None:
+                ev[1].record()
+
+        for _ in range(warmup):
+            iteration()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+        t0 = time.perf_counter()
+        for ev in evs:
+            iteration(ev)
+        torch.cuda.synchronize()
+        out[f"iteration_ms_overlap_{mode}"] = round((time.perf_counter() - t0) * 1e3 / iters, 3)
+        out[f"step_ms_overlap_{mode}"] = round(sum(a.elapsed_time(b) for a, b in evs) / iters, 3)
+        if mode == "on":
+            eng = next(iter(opt._muon_engines.values()))
+            out["matrices_staged_during_backward"] = len(eng._skip)
+        assert all(torch.isfinite(p).all() for p in pm[:2] + pa[:2])
+        del opt, pm, pa, xs, dys, coef, by_width
+        torch.cuda.empty_cache()
+    return out
+
+
 def summarize_kernels(per_label):
     out = {}
     gemm_work = gemm_ms = gemm_n = 0
@@ -313,6 +377,8 @@ def secondary(name, gates):
     if name != "ns32":
         g = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], use_graph=True)
         out["ms_per_step_graph_replay"] = round(g["ms_per_step"], 3)
+    if name == "gpt2-124m":
+        out["backward_overlap"] = run_backward_overlap(name)
     return out
 
 

@@ -231,6 +231,10 @@ int muon_amd_ns_gemm_noalloc(const MuonGemmDesc* descs_dev, const MuonTileJob* j
  *   u = nesterov ? lerp(grad, momentum, beta) : momentum       (lerp = torch's two-branch rule)
  * With mutate_grad != 0 and nesterov, u is also written back into grad as the reference does.
  * A matrix whose descriptor has momentum == NULL is only cast (u = grad).
+ * The launch may cover a run of the table instead of all of it (descs_dev + first, nmat = count,
+ * a prefix table of count + 1 entries that starts at 0): the sums of squares go to the slots
+ * part_begin + block-within-matrix either way.  A caller uses this to run the stage for one
+ * matrix as soon as its gradient exists, ahead of the rest of the step.
  * scalars_dev (here and in muon_amd_apply / muon_amd_adam): NULL, or device memory holding the
  * float arguments of the call in their order ({one_minus_beta, beta} here), which the kernel then
  * reads at run time in place of the by-value ones -- a launch recorded into a HIP graph can so

@@ -205,7 +205,9 @@ __global__ __launch_bounds__(EW_THREADS) void momentum_kernel(
                          ? momentum_block<uint16_t>(d, block_base, w, beta, nesterov, mutate_grad)
                          : momentum_block<float>(d, block_base, w, beta, nesterov, mutate_grad);
     const float total = block_sum_256(ss, red);
-    if (threadIdx.x == 0) d.partials[b] = total;
+    // slot = first slot of the matrix + block within the matrix: the same as the global block id
+    // in a launch over the whole table, and still right in a launch over part of it
+    if (threadIdx.x == 0) d.partials[d.part_begin + (b - prefix[mi])] = total;
 }
 
 // ------------------------------------------------------------------------------------------

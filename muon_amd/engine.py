@@ -85,6 +85,10 @@ class _ChunkRuntime:
                       chunk.aol_seg_prefix.view(np.uint8)]
             if chunk.poly_full_jobs is not None:
                 parts.append(chunk.poly_full_jobs.view(np.uint8))
+        # {0, blocks of matrix k} for every k: the prefix table of a momentum launch over matrix k alone
+        single = np.zeros((chunk.nmat, 2), dtype=np.int32)
+        single[:, 1] = np.diff(chunk.block_prefix)
+        parts.append(single.reshape(-1).view(np.uint8))
         offs, blob, cur = [], [], 0
         for p in parts:
             offs.append(cur)
@@ -108,8 +112,11 @@ class _ChunkRuntime:
         if chunk.aol:
             self.aol_ptr, self.aol_row_prefix_ptr, self.aol_seg_prefix_ptr = (b + o for o in offs[6:9])
             self.poly_full_jobs_ptr = b + offs[9] if chunk.poly_full_jobs is not None else None
+        self.single_prefix_ptr = b + offs[-1]
+        self.single_blocks = single[:, 1].tolist()
         self.mat_dev = None
         self.mat_key = None
+        self.mat_host = None
 
     def bind(self, grads, momenta, params, outs, scales, src_dtypes):
         """(Re)upload the matrix descriptors if any tensor address changed since the last call."""
@@ -130,12 +137,52 @@ class _ChunkRuntime:
                    "validate_mats")
         self.mat_dev = _upload(d, self.device, into=self.mat_dev)
         self.mat_key = key
+        self.mat_host = d
         self.src_dtypes = list(src_dtypes)
         self.present = [(bool(m), bool(p), bool(o)) for m, p, o in zip(momenta, params, outs)]
 
-    def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor, scalars_ptr=0):
+    def rebind_row(self, k, grad, momentum):
+        """Matrix k now has these gradient / momentum addresses: rewrite its descriptor in place
+        (on the current stream) and remember the addresses, so that the next `bind` with the same
+        ones uploads nothing."""
+        lib = _lib.load()
+        d = self.mat_host
+        d["grad"][k] = grad
+        d["momentum"][k] = momentum
+        _lib.check(lib.muon_amd_validate_mats(_lib.host_ptr(d), self.chunk.nmat,
+                                              _lib.host_ptr(self.chunk.block_prefix),
+                                              _lib.host_ptr(self.chunk.tile_prefix), self.chunk.tile),
+                   "validate_mats")
+        sz = _lib.MAT_DESC.itemsize
+        _upload(d[k:k + 1], self.device, into=self.mat_dev[k * sz:(k + 1) * sz])
+        g, m, *rest = self.mat_key
+        g, m = list(g), list(m)
+        g[k], m[k] = grad, momentum
+        self.mat_key = (tuple(g), tuple(m), *rest)
+
+    def momentum_of(self, k, one_minus_beta, beta, nesterov, mutate_grad, scalars_ptr=0, stream=None):
+        """The momentum launch over matrix k alone: on the current stream, or on `stream` (a raw
+        handle of a stream of this device, which must be the current device)."""
+        lib = _lib.load()
+
+        def call():
+            _lib.check(lib.muon_amd_momentum(
+                self.mat_dev.data_ptr() + k * _lib.MAT_DESC.itemsize, self.single_prefix_ptr + 8 * k, 1,
+                self.single_blocks[k], one_minus_beta, beta, int(nesterov), int(mutate_grad),
+                scalars_ptr or None, stream if stream is not None else _stream_ptr(self.device)), "momentum")
+
+        if stream is not None:          # per-launch events are recorded on the current stream only
+            call()
+            return
+        lay = self.chunk.layouts[k]
+        sz = 2 if self.src_dtypes[k] == _lib.SRC_BF16 else 4
+        _launch("momentum", lay.numel * (sz + 2 + (2 * sz if self.present[k][0] else 0)), call)
+
+    def run(self, one_minus_beta, beta, nesterov, mutate_grad, eps, lr, wd_factor, scalars_ptr=0,
+            momentum_done=frozenset()):
         """Enqueue the chunk's launches.  scalars_ptr: device address of {one_minus_beta, beta, lr,
-        wd_factor}, read by the kernels at run time in place of the by-value arguments."""
+        wd_factor}, read by the kernels at run time in place of the by-value arguments.
+        momentum_done: matrices (positions in the chunk) whose momentum stage already ran."""
         lib = _lib.load()
         c = self.chunk
         s = _stream_ptr(self.device)
@@ -157,9 +204,14 @@ class _ChunkRuntime:
             # (a fill kernel, recordable into a graph) keeps a launch that died half way from
             # poisoning every later step
             self.split_counters.zero_()
-        _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
-            mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
-            int(mutate_grad), sc_mom, s), "momentum"))
+        if not momentum_done:
+            _launch("momentum", mom_bytes, lambda: _lib.check(lib.muon_amd_momentum(
+                mats, self.block_prefix_ptr, c.nmat, c.nblocks, one_minus_beta, beta, int(nesterov),
+                int(mutate_grad), sc_mom, s), "momentum"))
+        else:
+            for k in range(c.nmat):
+                if k not in momentum_done:
+                    self.momentum_of(k, one_minus_beta, beta, nesterov, mutate_grad, scalars_ptr)
         norm_flags = flags | (_lib.NORM_UNIT if c.aol else 0)
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
             mats, c.nmat, eps, norm_flags, s), "norm_finalize"))
@@ -242,10 +294,32 @@ class MuonGroupEngine:
         assert base % 256 == 0
         self.runtimes = [_ChunkRuntime(c, base, self.device) for c in self.chunks]
         self._hyper = None
+        # matrices whose momentum stage may run ahead of the step: those of the first chunk (the
+        # later chunks reuse its workspace while the step runs); matrix index -> position in the chunk
+        self._early_pos = {lay.index: k for k, lay in enumerate(self.chunks[0].layouts)}
+        self._early_stream = None
+        self._early_events = {}
+        self._early_done = {}         # position -> gradient address the stage consumed
+        self._skip = frozenset()
 
     def prepare(self, grads, momenta, params, outs, scales, src_dtypes, *, beta, nesterov, mutate_grad,
                 eps, lr, weight_decay):
         """All list arguments are per matrix in the order of `shapes` (device addresses or 0)."""
+        if self._early_done:
+            # the stages enqueued by early_momentum since the last step: order them before what
+            # follows on this stream, and insist that they consumed the gradients of this step
+            torch.cuda.current_stream(self.device).wait_stream(self._early_stream)
+            layouts = self.chunks[0].layouts
+            done, self._early_done = self._early_done, {}
+            for k, used in done.items():
+                if grads[layouts[k].index] != used:
+                    raise _lib.MuonAmdError(
+                        f"the gradient of matrix {layouts[k].index} was replaced after its momentum stage ran "
+                        "during backward (overlap with backward needs the gradient tensors left alone "
+                        "between backward and step)")
+            self._skip = frozenset(done)
+        else:
+            self._skip = frozenset()
         for rt in self.runtimes:
             idx = [lay.index for lay in rt.chunk.layouts]
             rt.bind([grads[i] for i in idx], [momenta[i] for i in idx], [params[i] for i in idx],
@@ -261,13 +335,48 @@ class MuonGroupEngine:
     def structure_key(self):
         """What a recorded sequence of launches depends on besides device memory."""
         h = self._hyper
-        return (id(self), h["nesterov"], h["mutate_grad"], h["eps"])
+        return (id(self), h["nesterov"], h["mutate_grad"], h["eps"], self._skip)
 
     def enqueue(self, scalars_ptr: int = 0):
         h = self._hyper
-        for rt in self.runtimes:
+        for n, rt in enumerate(self.runtimes):
             rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
-                   h["wd_factor"], scalars_ptr=scalars_ptr)
+                   h["wd_factor"], scalars_ptr=scalars_ptr, momentum_done=self._skip if n == 0 else frozenset())
+
+    def early_momentum(self, i, grad, momentum, *, beta, nesterov, mutate_grad) -> bool:
+        """Run the first stage of matrix `i` (position in `shapes`) -- momentum, Nesterov blend,
+        bf16 cast, sums of squares -- now, on a side stream that first waits for everything enqueued
+        so far on the current stream (the work that produced the gradient), instead of inside the
+        step.  The next `prepare` joins the side stream, and that step's `enqueue` leaves the matrix
+        out of its momentum launch.  Meant to be called from a hook that fires during backward once
+        the gradient at address `grad` is complete.  Returns False, having done nothing, for a
+        matrix outside the first chunk or an engine that has not run a step yet."""
+        k = self._early_pos.get(i)
+        rt = self.runtimes[0]
+        if k is None or rt.mat_key is None:
+            return False
+        if k in self._early_done:
+            raise _lib.MuonAmdError(
+                f"matrix {i}: a second gradient arrived before step() (overlap with backward supports one "
+                "backward pass per step; the momentum buffer has already taken the first gradient)")
+        if self._early_stream is None:
+            self._early_stream = torch.cuda.Stream(self.device)
+        side = self._early_stream
+        ev = self._early_events.get(k)
+        if ev is None:
+            ev = self._early_events[k] = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        side.wait_event(ev)
+        moved = rt.mat_key[0][k] != grad or rt.mat_key[1][k] != momentum
+        if moved or torch.cuda.current_device() != self.device.index:
+            with torch.cuda.stream(side):
+                if moved:
+                    rt.rebind_row(k, grad, momentum)
+                rt.momentum_of(k, 1 - beta, beta, nesterov, mutate_grad)
+        else:       # the common case, kept cheap: this runs once per matrix inside backward
+            rt.momentum_of(k, 1 - beta, beta, nesterov, mutate_grad, stream=side.cuda_stream)
+        self._early_done[k] = grad
+        return True
 
     def run(self, grads, momenta, params, outs, scales, src_dtypes, **hyper):
         self.prepare(grads, momenta, params, outs, scales, src_dtypes, **hyper)

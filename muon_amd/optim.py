@@ -8,6 +8,8 @@ synchronises with the host.
 """
 from __future__ import annotations
 
+import weakref
+
 import torch
 
 from . import engine as _engine
@@ -26,8 +28,12 @@ def _world_size() -> int:
 class _MuonBase(torch.optim.Optimizer):
     """Shared machinery: engine caches and the two per-group update paths."""
 
-    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5", use_graph=False):
+    def _init_runtime(self, ns_rounding, mutate_grad, workspace_bytes, ns_variant="ns5", use_graph=False,
+                      overlap_backward=False):
         self._use_graph = bool(use_graph)
+        self._overlap_backward = bool(overlap_backward)
+        self._early_params = {}       # Muon parameter -> (engine, first matrix, matrices, group), set by each step
+        self._install_overlap_hooks()
         if ns_variant not in ("ns5", "aol4", "aol4_rows"):
             raise ValueError(f"ns_variant must be 'ns5', 'aol4' or 'aol4_rows', got {ns_variant!r}")
         self._ns_variant = ns_variant
@@ -42,7 +48,58 @@ class _MuonBase(torch.optim.Optimizer):
         self._writebacks = []         # (destination, contiguous copy) pairs to copy back after the launches
         self._keepalive = []          # temporaries whose addresses the pending launches use
 
-    _RUNTIME_OPTIONS = ("_ns_rounding", "_mutate_grad", "_workspace_bytes", "_ns_variant", "_use_graph")
+    _RUNTIME_OPTIONS = ("_ns_rounding", "_mutate_grad", "_workspace_bytes", "_ns_variant", "_use_graph",
+                        "_overlap_backward")
+
+    # ---- overlap with backward: the first Muon stage of a matrix runs when its gradient is ready ----
+    def _install_overlap_hooks(self):
+        for h in getattr(self, "_hook_handles", []):
+            h.remove()
+        self._hook_handles = []
+        self._hooked = set()
+        if self._overlap_backward:
+            for group in self.param_groups:
+                self._hook_group(group)
+
+    def _hook_group(self, group):
+        if not group.get("use_muon", True):
+            return
+        ref = weakref.ref(self)           # the parameters must not keep the optimizer alive
+
+        def grad_ready(p):
+            opt = ref()
+            if opt is not None:
+                opt._grad_ready(p)
+
+        for p in group["params"]:
+            if isinstance(p, torch.Tensor) and p.requires_grad and p.is_leaf and id(p) not in self._hooked:
+                self._hook_handles.append(p.register_post_accumulate_grad_hook(grad_ready))
+                self._hooked.add(id(p))
+
+    def add_param_group(self, param_group):
+        super().add_param_group(param_group)
+        if getattr(self, "_overlap_backward", False):
+            self._hook_group(self.param_groups[-1])
+
+    @torch.no_grad()
+    def _grad_ready(self, p):
+        """Autograd has finished accumulating p.grad (post-accumulate-grad hook).  Once a step has
+        built the group's engine, enqueue the matrix's momentum stage on the engine's side stream;
+        step() then skips it.  Anything out of the ordinary (no engine yet, strided tensors, a
+        gradient of another dtype) is left to step()."""
+        info = self._early_params.get(p)
+        if info is None:
+            return
+        eng, first, count, group = info
+        g, m = p.grad, self.state[p].get("momentum_buffer")
+        if (g is None or m is None or g.is_sparse or g.dtype != p.dtype or m.dtype != p.dtype or
+                m.shape != p.shape or g.device != p.device or m.device != p.device or
+                not (g.is_contiguous() and m.is_contiguous() and p.is_contiguous())):
+            return
+        stride = (p.numel() // count) * p.element_size()
+        for k in range(count):
+            eng.early_momentum(first + k, g.data_ptr() + k * stride, m.data_ptr() + k * stride,
+                               beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad)
 
     def __getstate__(self):
         # torch's Optimizer pickles defaults/state/param_groups only; the keyword-only options of
@@ -58,7 +115,7 @@ class _MuonBase(torch.optim.Optimizer):
         super().__setstate__(state)
         if opts is not None:
             self._init_runtime(opts["_ns_rounding"], opts["_mutate_grad"], opts["_workspace_bytes"],
-                               opts["_ns_variant"], opts["_use_graph"])
+                               opts["_ns_variant"], opts["_use_graph"], opts.get("_overlap_backward", False))
         elif not hasattr(self, "_muon_engines"):
             self._init_runtime("reference", False, None)
 
@@ -101,6 +158,7 @@ class _MuonBase(torch.optim.Optimizer):
         if not params:
             return
         grads, moms, ptrs, shapes, scales, dtypes, writebacks, keep = [], [], [], [], [], [], [], []
+        spans = []                                # (parameter, first matrix, matrices) of plain row-major parameters
         for p in params:
             self._check_param(p)
             assert p.ndim >= 2                    # muon.py:275 (reached through muon.py:13)
@@ -118,6 +176,8 @@ class _MuonBase(torch.optim.Optimizer):
                 rows, cols = p.shape[-2:]
                 batch = p.numel() // (rows * cols)
             scale = max(1, p.size(-2) / p.size(-1)) ** 0.5             # muon.py:14
+            if g is p.grad and pc is p and m is state["momentum_buffer"]:
+                spans.append((p, len(shapes), batch))
             for k in range(batch):
                 off = k * rows * cols * p.element_size()
                 shapes.append((rows, cols))
@@ -143,6 +203,11 @@ class _MuonBase(torch.optim.Optimizer):
         self._pending.append(eng)
         self._writebacks += writebacks
         self._keepalive.append(keep)
+        if self._overlap_backward:
+            for p in params:
+                self._early_params.pop(p, None)
+            for p, first, count in spans:
+                self._early_params[p] = (eng, first, count, group)
 
     def _adam_group_step(self, gi, group):
         by_step, writebacks = {}, []
@@ -220,14 +285,21 @@ class SingleDeviceMuon(_MuonBase):
     zeropower_via_aol4), use_graph
     (record every launch of a step -- all Muon groups and all Adam groups on a device -- into one
     HIP graph once and replay it every step; tensor addresses and hyper-parameters are read from
-    device memory, so gradients may be reallocated and learning rates scheduled between steps).
+    device memory, so gradients may be reallocated and learning rates scheduled between steps),
+    overlap_backward (post-accumulate-grad hooks on the Muon parameters run a matrix's first stage
+    -- momentum, Nesterov blend, bf16 cast, sums of squares -- on a side stream as soon as backward
+    has produced its gradient, and step() skips it; from the second step on, for the matrices of
+    the first workspace chunk.  It needs exactly one backward pass per step and gradients that
+    nothing touches between backward and step -- no accumulation over micro-batches, no clipping;
+    a second gradient or a replaced gradient tensor raises).
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
-                 mutate_grad=False, workspace_bytes=None, ns_variant="ns5", use_graph=False):
+                 mutate_grad=False, workspace_bytes=None, ns_variant="ns5", use_graph=False,
+                 overlap_backward=False):
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum)
         super().__init__(params, defaults)
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph, overlap_backward)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -279,10 +351,10 @@ class SingleDeviceMuonWithAuxAdam(_MuonBase):
     _SORT_MUON = False
 
     def __init__(self, param_groups, *, ns_rounding="reference", mutate_grad=False, workspace_bytes=None,
-                 ns_variant="ns5", use_graph=False):
+                 ns_variant="ns5", use_graph=False, overlap_backward=False):
         _fill_aux_adam_groups(param_groups, self._SORT_MUON)
         super().__init__(param_groups, dict())
-        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph)
+        self._init_runtime(ns_rounding, mutate_grad, workspace_bytes, ns_variant, use_graph, overlap_backward)
 
     @torch.no_grad()
     def step(self, closure=None):

@@ -1,0 +1,135 @@
+"""overlap_backward=True on the GPU: post-accumulate-grad hooks run a matrix's first Muon stage
+(muon.py:9-10 and the cast of muon.py:277) on a side stream while autograd is still producing
+the other gradients, and step() skips that stage for those matrices.  The result must be the
+bits of the plain step, the step itself must match the oracle, and the two misuse cases the
+option cannot support must raise instead of corrupting the momentum buffers.
+"""
+import pytest
+import torch
+
+from oracle import muon_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def M():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need an MI355X; torch.cuda.is_available() is False")
+    import muon_amd
+    from muon_amd import _lib
+    _lib.load()
+    return muon_amd
+
+
+SHAPES = [(768, 768), (256, 640), (640, 256), (3, 128, 192), (16, 8, 3, 3), (130, 300)]
+
+
+def _params(seed, device="cuda"):
+    torch.manual_seed(seed)
+    return [torch.nn.Parameter((torch.randn(*s) * 0.02).to(device)) for s in SHAPES]
+
+
+def _inputs(params, seed):
+    """Per parameter a layer input x and an output gradient dy: the loss below makes autograd produce
+    every weight gradient as the matrix product x^T . dy of a linear layer's backward (full rank:
+    512 rows)."""
+    gen = torch.Generator().manual_seed(seed)
+    out = []
+    for p in params:
+        rows, cols = (p.shape[0], p.numel() // p.shape[0]) if p.ndim == 4 else p.shape[-2:]
+        lead = tuple(p.shape[:-2]) if p.ndim == 3 else ()
+        out.append((torch.randn(*lead, 512, rows, generator=gen) * 1e-2, torch.randn(*lead, 512, cols, generator=gen) * 1e-2))
+    return out
+
+
+def _loss(params, xs):
+    total = 0.0
+    for p, (x, dy) in zip(params, xs):
+        w = p.reshape(p.shape[0], -1) if p.ndim == 4 else p
+        total = total + ((x.to(p.device) @ w) * dy.to(p.device)).sum()
+    return total
+
+
+def _make(M, params, gain, **kw):
+    return M.SingleDeviceMuonWithAuxAdam(
+        [dict(params=params, use_muon=True, lr=0.02, weight_decay=0.01),
+         dict(params=[gain], use_muon=False, lr=3e-4, weight_decay=0.0)], **kw)
+
+
+@pytest.mark.parametrize("use_graph,cap", [(False, None), (True, None), (False, 3 << 20)])
+def test_overlap_with_backward_equals_the_plain_step(M, use_graph, cap):
+    pa, pb = _params(77), _params(77)
+    ga, gb = (torch.nn.Parameter(torch.ones(40, device="cuda")) for _ in range(2))
+    plain = _make(M, pa, ga, workspace_bytes=cap)
+    early = _make(M, pb, gb, workspace_bytes=cap, use_graph=use_graph, overlap_backward=True)
+    skipped = []
+    for step in range(5):
+        xs = _inputs(pa, 100 + step)
+        if step == 3:        # the hooks read the group's momentum when they fire: change it before backward
+            plain.param_groups[0]["momentum"] = early.param_groups[0]["momentum"] = 0.9
+        for opt, params, gain in ((plain, pa, ga), (early, pb, gb)):
+            opt.zero_grad(set_to_none=(step % 2 == 0))      # reallocated and reused gradient tensors
+            (_loss(params, xs) + (gain * gain).sum()).backward()
+        plain.step()
+        early.step()
+        eng = next(iter(early._muon_engines.values()))
+        skipped.append(len(eng._skip))
+        torch.cuda.synchronize()
+        for a, b in zip(pa + [ga], pb + [gb]):
+            assert torch.equal(a.detach(), b.detach()), (step, tuple(a.shape))
+        for a, b in zip(pa, pb):
+            assert torch.equal(plain.state[a]["momentum_buffer"], early.state[b]["momentum_buffer"]), (step, tuple(a.shape))
+    eng = next(iter(early._muon_engines.values()))
+    first_chunk = len(eng.chunks[0].layouts)
+    # the first step builds the engine; from the second on, every matrix of the first chunk is done early
+    assert skipped[0] == 0 and all(s == first_chunk for s in skipped[1:]), (skipped, first_chunk)
+    if cap is None:
+        assert first_chunk == len(eng.shapes) == len(SHAPES) + 2          # the 3-D parameter is three matrices
+    else:
+        assert len(eng.runtimes) > 1 and first_chunk < len(eng.shapes)
+
+
+def test_overlapped_step_matches_the_oracle(M):
+    gpu = _params(78)
+    cpu = [torch.nn.Parameter(p.detach().cpu().clone()) for p in gpu]
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, overlap_backward=True)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01)
+    for step in range(3):
+        xs = _inputs(gpu, 200 + step)
+        for opt, params in ((og, gpu), (oc, cpu)):
+            opt.zero_grad(set_to_none=True)
+            _loss(params, xs).backward()
+        og.step()
+        oc.step()
+        for pc, pg in zip(cpu, gpu):
+            tol = (1e-3 if pc.ndim == 2 else 3e-3) * (step + 1) ** 0.5
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= tol, (step, tuple(pc.shape))
+    assert len(next(iter(og._muon_engines.values()))._skip) == len(SHAPES) + 2       # the 3-D parameter is three matrices
+
+
+def test_overlap_refuses_a_second_backward_and_a_replaced_gradient(M):
+    from muon_amd._lib import MuonAmdError
+    params = _params(79)
+    opt = M.SingleDeviceMuon(params, overlap_backward=True)
+    xs = _inputs(params, 300)
+    _loss(params, xs).backward()
+    opt.step()                                   # builds the engine; hooks act from now on
+    opt.zero_grad(set_to_none=True)
+    _loss(params, xs).backward()
+    with pytest.raises(MuonAmdError, match="second gradient"):
+        _loss(params, xs).backward()             # accumulation over micro-batches
+    opt.step()                                   # consumes what the first of the two passes started
+    torch.cuda.synchronize()
+    opt.zero_grad(set_to_none=True)
+    _loss(params, xs).backward()
+    params[0].grad = params[0].grad.clone()      # what a clipping routine that reallocates would do
+    with pytest.raises(MuonAmdError, match="replaced"):
+        opt.step()
+    torch.cuda.synchronize()
+    # the optimizer is usable again afterwards
+    opt.zero_grad(set_to_none=True)
+    _loss(params, xs).backward()
+    opt.step()
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(p).all() for p in params)

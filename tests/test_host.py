@@ -350,3 +350,26 @@ def test_header_is_plain_c_and_field_offsets_match_the_binding(tmp_path):
         assert got[(name, "size")] == dt.itemsize
         for field in dt.names:
             assert got[(name, field)] == dt.fields[field][1], (name, field)
+
+
+def test_overlap_backward_option_installs_hooks_and_survives_copies():
+    """overlap_backward=True registers one post-accumulate-grad hook per Muon parameter (none on
+    Adam parameters), new groups get theirs, copies of the optimizer re-register on their own
+    parameters, and before the first step the hooks do nothing (there is no engine yet)."""
+    import copy
+    import muon_amd as M
+    w = [torch.nn.Parameter(torch.randn(8, 4)), torch.nn.Parameter(torch.randn(4, 8))]
+    gain = torch.nn.Parameter(torch.ones(4))
+    opt = M.SingleDeviceMuonWithAuxAdam([dict(params=w, use_muon=True), dict(params=[gain], use_muon=False)],
+                                        overlap_backward=True)
+    assert len(opt._hook_handles) == 2 and opt._overlap_backward
+    (w[0].sum() + w[1].sum() + gain.sum()).backward()          # hooks fire: nothing to do yet, no GPU touched
+    assert all(p.grad is not None for p in w) and not opt._early_params
+    extra = torch.nn.Parameter(torch.randn(4, 4))
+    opt.add_param_group(dict(params=[extra], use_muon=True, lr=0.02, momentum=0.95, weight_decay=0))
+    assert len(opt._hook_handles) == 3
+    dup = copy.deepcopy(opt)
+    assert dup._overlap_backward and len(dup._hook_handles) == 3
+    assert all(p._post_accumulate_grad_hooks for g in dup.param_groups if g["use_muon"] for p in g["params"])
+    plain = M.SingleDeviceMuon([torch.nn.Parameter(torch.randn(4, 4))])
+    assert not plain._overlap_backward and plain._hook_handles == []
