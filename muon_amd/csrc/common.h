@@ -37,9 +37,16 @@ __device__ __forceinline__ float bf2f(uint16_t h) {
 // fp32 value rounded through bf16.
 __device__ __forceinline__ float round_bf(float f) { return bf2f(f2bf(f)); }
 
+// Two fp32 values rounded to bf16 and packed (lo in bits 0-15): one v_cvt_pk_bf16_f32.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
-    return static_cast<uint32_t>(f2bf(lo)) | (static_cast<uint32_t>(f2bf(hi)) << 16);
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+// The halves of such a pair as fp32.
+__device__ __forceinline__ float bf_lo(uint32_t p) { return __uint_as_float(p << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
 
 // torch's lerp (ATen/native/Lerp.h): two algebraically equal forms chosen by |weight|.
 __device__ __forceinline__ float lerp_torch(float start, float end, float w) {

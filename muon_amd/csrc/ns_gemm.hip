@@ -106,6 +106,18 @@ __device__ __forceinline__ f32x16 tile_transpose_bf16(const float (&v)[16], bf16
     return z;
 }
 
+// The same for a tile already packed two bf16 per register (p[k] = values 2k, 2k+1).
+__device__ __forceinline__ f32x16 tile_transpose_packed(const uint32_t (&p)[8], bf16x8 id0, bf16x8 id1) {
+    const bf16x8 f0 = __builtin_bit_cast(bf16x8, u32x4{p[0], p[1], p[2], p[3]});
+    const bf16x8 f1 = __builtin_bit_cast(bf16x8, u32x4{p[4], p[5], p[6], p[7]});
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f0, id0, z, 0, 0, 0);
+    z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f1, id1, z, 0, 0, 0);
+    return z;
+}
+
 // bf16(gamma * x) for 8 packed bf16 values.
 __device__ __forceinline__ u32x4 scale_bf16x8(u32x4 v, float gamma) {
     u32x4 r;
@@ -281,14 +293,60 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
         float rowpart = 0.f;  // ROWSUM: |o| summed along this lane's 32 of the strip's 64 columns
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
-            f32x16 u;
             if (round_terms) {
-                float t1[16];
+                // Every term rounded to bf16 as the reference's tensor expressions round.  Values
+                // stay packed two bf16 per register from the conversion that rounds them: the pairs
+                // are what the transposing MFMAs, the staging stores and the next conversion take.
+                uint32_t p1[8];       // bf16(alpha * acc), accumulator layout
 #pragma unroll
-                for (int i = 0; i < 16; ++i) t1[i] = round_bf(alpha * acc[a][b][i]);
-                u = tile_transpose_bf16(t1, id0, id1);
-            } else {
-                // keep ~16 mantissa bits: transpose a bf16 head and a bf16 tail and add them
+                for (int k = 0; k < 8; ++k) p1[k] = pack2bf(alpha * acc[a][b][2 * k], alpha * acc[a][b][2 * k + 1]);
+                const f32x16 u = tile_transpose_packed(p1, id0, id1);
+                uint32_t po[8];       // o = bf16(u + bf16(beta * D)), row-owning layout
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (HAS_D) {
+                        const uint32_t t01 = pack2bf(beta * bf_lo(dv[a][b][q].x), beta * bf_hi(dv[a][b][q].x));
+                        const uint32_t t23 = pack2bf(beta * bf_lo(dv[a][b][q].y), beta * bf_hi(dv[a][b][q].y));
+                        po[2 * q] = pack2bf(u[4 * q] + bf_lo(t01), u[4 * q + 1] + bf_hi(t01));
+                        po[2 * q + 1] = pack2bf(u[4 * q + 2] + bf_lo(t23), u[4 * q + 3] + bf_hi(t23));
+                    } else {          // u holds bf16 values: exact
+                        po[2 * q] = pack2bf(u[4 * q], u[4 * q + 1]);
+                        po[2 * q + 1] = pack2bf(u[4 * q + 2], u[4 * q + 3]);
+                    }
+                    if constexpr (ROWSUM) {       // one term after the other, in column order
+                        rowpart += fabsf(bf_lo(po[2 * q]));
+                        rowpart += fabsf(bf_hi(po[2 * q]));
+                        rowpart += fabsf(bf_lo(po[2 * q + 1]));
+                        rowpart += fabsf(bf_hi(po[2 * q + 1]));
+                    }
+                    if (do_d)
+                        *reinterpret_cast<u32x2*>(stage + lr * DROW + (b * 32 + 8 * q + 4 * g) * 2) =
+                            u32x2{po[2 * q], po[2 * q + 1]};
+                }
+                if (do_t) {
+                    if (HAS_D) {
+                        const f32x16 w = tile_transpose_packed(po, id0, id1);
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) ot[b][k] = pack2bf(w[2 * k], w[2 * k + 1]);
+                    } else {
+                        // without an addend o is the transposed t1, and its transpose is t1 again
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) ot[b][k] = p1[k];
+                        if constexpr (ROWSUM) {
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) {
+                                colsum[b] += fabsf(bf_lo(p1[k]));
+                                colsum[b] += fabsf(bf_hi(p1[k]));
+                            }
+                        }
+                    }
+                }
+                continue;
+            }
+            // One rounding per output: keep ~16 mantissa bits of alpha * acc through the transpose by
+            // moving a bf16 head and a bf16 tail and adding them.
+            f32x16 u;
+            {
                 float hi[16], lo[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -306,16 +364,14 @@ __device__ __forceinline__ void ns_epilogue_strips(f32x16 (&acc)[TM][TN], const 
             for (int q = 0; q < 4; ++q) {
                 float dd[4] = {0.f, 0.f, 0.f, 0.f};
                 if (HAS_D) {
-                    dd[0] = __uint_as_float(dv[a][b][q].x << 16);
-                    dd[1] = __uint_as_float(dv[a][b][q].x & 0xffff0000u);
-                    dd[2] = __uint_as_float(dv[a][b][q].y << 16);
-                    dd[3] = __uint_as_float(dv[a][b][q].y & 0xffff0000u);
+                    dd[0] = bf_lo(dv[a][b][q].x);
+                    dd[1] = bf_hi(dv[a][b][q].x);
+                    dd[2] = bf_lo(dv[a][b][q].y);
+                    dd[3] = bf_hi(dv[a][b][q].y);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float t2 = HAS_D ? beta * dd[e] : 0.f;
-                    if (round_terms) t2 = round_bf(t2);
-                    o[4 * q + e] = round_bf(u[4 * q + e] + t2);
+                    o[4 * q + e] = round_bf(u[4 * q + e] + (HAS_D ? beta * dd[e] : 0.f));
                     if constexpr (ROWSUM) rowpart += fabsf(o[4 * q + e]);
                 }
                 if (do_d) {
