@@ -154,7 +154,8 @@ def correctness_gates(name):
 # ------------------------------------------------------------------------------------------
 # GPU leg
 # ------------------------------------------------------------------------------------------
-def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False, realloc_grads=False):
+def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False, realloc_grads=False,
+                           launch_events=True):
     import muon_amd
     from muon_amd import engine
 
@@ -198,8 +199,10 @@ def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_grap
     torch.cuda.synchronize()
 
     # timed region: exactly `steps` steps back to back, one synchronisation on either side; a pair
-    # of HIP events on the launch stream brackets every kernel launch inside it
-    engine.PROFILE = None if use_graph else []      # a replayed graph has no per-launch events
+    # of HIP events on the launch stream brackets every kernel launch inside it (recording them
+    # costs the host a few microseconds per launch, which a step of a small model notices:
+    # launch_events=False times the same region without them)
+    engine.PROFILE = None if (use_graph or not launch_events) else []      # a replayed graph has no per-launch events
     t0 = time.perf_counter()
     for _ in range(steps):
         one_step()
@@ -375,6 +378,10 @@ def secondary(name, gates):
                 "ns_frac_of_peak": round(gw / gms / 1e9 / PEAK_BF16_TFLOPS, 4), "gemm_launches": gn,
                 "avg_gemm_launch_ms": round(gms / gn, 4)})
     if name != "ns32":
+        # the same steps without the per-launch events: what a training loop sees
+        plain = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], launch_events=False)
+        out["ms_per_step_with_launch_events"] = out["ms_per_step"]
+        out["ms_per_step"] = round(plain["ms_per_step"], 3)
         g = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], use_graph=True)
         out["ms_per_step_graph_replay"] = round(g["ms_per_step"], 3)
     if name == "gpt2-124m":
@@ -626,6 +633,11 @@ def main():
         },
         "kernels": rounded(kernels),
     }
+    if args.workload != "llama3-8b" and not args.realloc_grads:
+        # a small model's step is short enough for the host cost of the launch events to show
+        plain = run_optimizer_workload(args.workload, steps, warmup, seed=1234 + 4, ns_variant=args.ns_variant,
+                                       launch_events=False)
+        line["ms_per_step_without_launch_events"] = round(plain["ms_per_step"], 3)
     if not args.no_extra and args.workload == "llama3-8b":
         line["gpt2_124m"] = secondary("gpt2-124m", not args.no_gates)
         line["ns32"] = secondary("ns32", not args.no_gates)
