@@ -291,7 +291,9 @@ class SingleDeviceMuon(_MuonBase):
     has produced its gradient, and step() skips it; from the second step on, for the matrices of
     the first workspace chunk.  It needs exactly one backward pass per step and gradients that
     nothing touches between backward and step -- no accumulation over micro-batches, no clipping;
-    a second gradient or a replaced gradient tensor raises).
+    a second gradient or a replaced gradient tensor raises.  The momentum buffers take the gradient
+    when backward produces it: a step() that is then skipped, as a loss scaler does after an
+    overflow, leaves them updated all the same).
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",
