@@ -119,6 +119,25 @@ def matrix_workspace_bytes(rows: int, cols: int, unit: int) -> int:
             3 * _round_up(mp * (mp + LD_PAD) * 2, _ALIGN))
 
 
+def matrix_scratch_bytes(rows: int, cols: int, tile_class: int, aol: bool) -> int:
+    """Upper bound of what a matrix adds to a chunk's workspace besides its six bf16 buffers: the
+    sums of squares of its elementwise blocks, its denominator, the fp32 slots of its split
+    reductions and, for the AOL variants, its row scales and partial row sums (each rounded up to
+    the alignment: the chunk rounds the first two once for all its matrices)."""
+    unit = pad_unit(tile_class)
+    tr, tc = TILE_DIMS[tile_class]
+    m, n = min(rows, cols), max(rows, cols)
+    mp, np_ = _round_up(m, unit), _round_up(n, unit)
+    total = _round_up(-(-rows * cols // EW_BLOCK_ELEMS) * 4, _ALIGN) + _ALIGN
+    nsplit = split_factor(mp, np_)
+    if nsplit > 1:
+        tiles = (mp // tr) * (mp // tr + 1) // 2 * (tr // tc) if tr != tc else (mp // tr) * (mp // tr + 1) // 2
+        total += _round_up(tiles * nsplit * tr * tc * 4, _ALIGN)
+    if aol:
+        total += _round_up(mp * 4, _ALIGN) + _round_up(mp * (mp // ROWSUM_SLOT) * 4, _ALIGN)
+    return total
+
+
 @lru_cache(maxsize=256)
 def _tile_order(mt: int, nt: int, sym: bool, ratio: int, super_i: int, super_j: int):
     """Tiles of an mt x nt grid in super-block order.  `ratio` = tile rows / tile cols; with sym
@@ -363,8 +382,9 @@ class ChunkPlan:
 
 
 def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5"):
-    """Split matrices [(rows, cols), ...] into chunks of one tile class each whose workspace stays
-    under `workspace_cap` bytes (a single matrix larger than the cap gets a chunk of its own).
+    """Split matrices [(rows, cols), ...] into chunks of one tile class each whose workspace (the bf16
+    buffers and the scratch beside them) stays under `workspace_cap` bytes (a single matrix larger
+    than the cap gets a chunk of its own).
     Same-shape matrices are kept together so that their tiles batch into full waves of the GPU."""
     order = sorted(range(len(shapes)),
                    key=lambda i: (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]),
@@ -373,7 +393,8 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
     for i in order:
         rows, cols = shapes[i]
         tc = tile_class_for(min(rows, cols))
-        need = matrix_workspace_bytes(rows, cols, pad_unit(tc))
+        need = (matrix_workspace_bytes(rows, cols, pad_unit(tc)) +
+                matrix_scratch_bytes(rows, cols, tc, variant in ("aol4", "aol4_rows")))
         if cur and (tc != cur_class or cur_bytes + need > workspace_cap):
             chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding, variant))
             cur, cur_bytes = [], 0

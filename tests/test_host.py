@@ -57,6 +57,57 @@ def test_entry_points_reject_bad_arguments_without_a_gpu():
 SHAPES = [(768, 3072), (3072, 768), (768, 768), (4096, 4096), (64, 216), (16384, 128), (5, 3), (1024, 4096)]
 
 
+def _check_chunk(lib, c):
+    """Tables of one chunk: accepted by the library's validators, every tile of every product
+    covered exactly once, workspace regions disjoint and inside the workspace."""
+    T = c.tile
+    assert all(plan.tile_class_for(l.m) == c.tile_class for l in c.layouts)
+    g = c.gemm_descs(1 << 20)
+    for ph in range(5):
+        jobs = c.syrk_jobs if ph == plan.PH_SYRK else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
+        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class,
+                                        c.split_slots if ph == plan.PH_SYRK else 0)
+        assert rc == 0, lib.muon_amd_last_error()
+    TR, TC = c.tile_rows, c.tile_cols
+    for k, l in enumerate(c.layouts):
+        mt, nt, ratio = l.mp // TR, l.np_ // TC, TR // TC
+        sj = c.sym_jobs[c.sym_jobs["desc"] == k]
+        got = sorted(zip((sj["i0"] // TR).tolist(), (sj["j0"] // TC).tolist()))
+        assert got == [(i, j) for i in range(mt) for j in range(i * ratio, l.mp // TC)]
+        assert np.array_equal(sj["diag"], (sj["i0"] // TR == sj["j0"] // TR).astype(np.int32))
+        # direct tiles plus mirrors of the off-diagonal-block tiles cover the matrix exactly once
+        cover = np.zeros((l.mp // TC, l.mp // TC), dtype=int)
+        for i0, j0, dg in zip(sj["i0"].tolist(), sj["j0"].tolist(), sj["diag"].tolist()):
+            cover[i0 // TC:(i0 + TR) // TC, j0 // TC] += 1
+            if not dg:
+                cover[j0 // TC, i0 // TC:(i0 + TR) // TC] += 1
+        assert (cover == 1).all()
+        fj = c.full_jobs[c.full_jobs["desc"] == k]
+        got = sorted(zip((fj["i0"] // TR).tolist(), (fj["j0"] // TC).tolist()))
+        assert got == [(i, j) for i in range(mt) for j in range(nt)]
+        assert l.mp % T == 0 and l.np_ % T == 0 and l.mp >= l.m and l.np_ >= l.n
+        assert l.wide == (l.rows <= l.cols)
+    # workspace regions do not overlap and stay inside the chunk's workspace
+    regions = []
+    for l in c.layouts:
+        size = {"X": l.mp * l.ldn * 2, "XT0": l.np_ * l.ldm * 2, "XT1": l.np_ * l.ldm * 2,
+                "A": l.mp * l.ldm * 2, "B": l.mp * l.ldm * 2, "CA": l.mp * l.ldm * 2}
+        for name in ("X", "XT0", "XT1", "A", "B", "CA"):
+            regions.append((l.off[name], l.off[name] + size[name]))
+    regions += [(c.off_partials, c.off_partials + 4 * c.nblocks), (c.off_denoms, c.off_denoms + 4 * c.nmat)]
+    regions.sort()
+    assert all(a[1] <= b[0] for a, b in zip(regions, regions[1:])) and regions[-1][1] <= c.workspace_bytes
+    assert all(r[0] % 256 == 0 for r in regions)
+    md = c.mat_descs(1 << 20)
+    md["grad"] = 4096
+    md["out"] = 8192
+    rc = lib.muon_amd_validate_mats(_lib.host_ptr(md), c.nmat, _lib.host_ptr(c.block_prefix),
+                                    _lib.host_ptr(c.tile_prefix), c.tile)
+    assert rc == 0, lib.muon_amd_last_error()
+
+
+
+
 @pytest.mark.parametrize("ref", [True, False])
 def test_plans_validate_and_cover_every_tile_once(ref):
     lib = _lib.load()
@@ -64,50 +115,38 @@ def test_plans_validate_and_cover_every_tile_once(ref):
     seen = sorted(l.index for c in chunks for l in c.layouts)
     assert seen == list(range(len(SHAPES)))
     for c in chunks:
-        T = c.tile
-        assert all(plan.tile_class_for(l.m) == c.tile_class for l in c.layouts)
-        g = c.gemm_descs(1 << 20)
-        for ph in range(5):
-            jobs = c.syrk_jobs if ph == plan.PH_SYRK else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
-            rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class,
-                                            c.split_slots if ph == plan.PH_SYRK else 0)
-            assert rc == 0, lib.muon_amd_last_error()
-        TR, TC = c.tile_rows, c.tile_cols
-        for k, l in enumerate(c.layouts):
-            mt, nt, ratio = l.mp // TR, l.np_ // TC, TR // TC
-            sj = c.sym_jobs[c.sym_jobs["desc"] == k]
-            got = sorted(zip((sj["i0"] // TR).tolist(), (sj["j0"] // TC).tolist()))
-            assert got == [(i, j) for i in range(mt) for j in range(i * ratio, l.mp // TC)]
-            assert np.array_equal(sj["diag"], (sj["i0"] // TR == sj["j0"] // TR).astype(np.int32))
-            # direct tiles plus mirrors of the off-diagonal-block tiles cover the matrix exactly once
-            cover = np.zeros((l.mp // TC, l.mp // TC), dtype=int)
-            for i0, j0, dg in zip(sj["i0"].tolist(), sj["j0"].tolist(), sj["diag"].tolist()):
-                cover[i0 // TC:(i0 + TR) // TC, j0 // TC] += 1
-                if not dg:
-                    cover[j0 // TC, i0 // TC:(i0 + TR) // TC] += 1
-            assert (cover == 1).all()
-            fj = c.full_jobs[c.full_jobs["desc"] == k]
-            got = sorted(zip((fj["i0"] // TR).tolist(), (fj["j0"] // TC).tolist()))
-            assert got == [(i, j) for i in range(mt) for j in range(nt)]
-            assert l.mp % T == 0 and l.np_ % T == 0 and l.mp >= l.m and l.np_ >= l.n
-            assert l.wide == (l.rows <= l.cols)
-        # workspace regions do not overlap and stay inside the chunk's workspace
-        regions = []
-        for l in c.layouts:
-            size = {"X": l.mp * l.ldn * 2, "XT0": l.np_ * l.ldm * 2, "XT1": l.np_ * l.ldm * 2,
-                    "A": l.mp * l.ldm * 2, "B": l.mp * l.ldm * 2, "CA": l.mp * l.ldm * 2}
-            for name in ("X", "XT0", "XT1", "A", "B", "CA"):
-                regions.append((l.off[name], l.off[name] + size[name]))
-        regions += [(c.off_partials, c.off_partials + 4 * c.nblocks), (c.off_denoms, c.off_denoms + 4 * c.nmat)]
-        regions.sort()
-        assert all(a[1] <= b[0] for a, b in zip(regions, regions[1:])) and regions[-1][1] <= c.workspace_bytes
-        assert all(r[0] % 256 == 0 for r in regions)
-        md = c.mat_descs(1 << 20)
-        md["grad"] = 4096
-        md["out"] = 8192
-        rc = lib.muon_amd_validate_mats(_lib.host_ptr(md), c.nmat, _lib.host_ptr(c.block_prefix),
-                                        _lib.host_ptr(c.tile_prefix), c.tile)
-        assert rc == 0, lib.muon_amd_last_error()
+        _check_chunk(lib, c)
+
+
+def test_random_parameter_lists_plan_into_valid_tables():
+    """Seeded random lists of shapes (tiny, around the tile edges, tall, wide), random workspace
+    caps, both roundings and the AOL variants: every chunk passes the same checks."""
+    import random
+    lib = _lib.load()
+    rng = random.Random(7)
+    edge = [1, 2, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 767, 768, 1023, 1024, 1025, 2048, 4096]
+
+    def dim():
+        k = rng.random()
+        return rng.randint(1, 70) if k < 0.3 else rng.choice(edge) if k < 0.7 else rng.randint(64, 5000)
+
+    for case in range(60):
+        shapes = [(dim(), dim()) for _ in range(rng.randint(1, 12))]
+        variant = rng.choice(["ns5", "ns5", "aol4", "aol4_rows"])
+        aol = variant != "ns5"
+        biggest = max(plan.matrix_workspace_bytes(r, c, plan.pad_unit(plan.tile_class_for(min(r, c)))) +
+                      plan.matrix_scratch_bytes(r, c, plan.tile_class_for(min(r, c)), aol) for r, c in shapes)
+        cap = max(biggest, rng.choice([1 << 20, 16 << 20, 256 << 20, 1 << 34]))
+        chunks = plan.plan_chunks(shapes, 5, rng.random() < 0.5, cap, variant)
+        assert sorted(l.index for c in chunks for l in c.layouts) == list(range(len(shapes))), (case, shapes)
+        for c in chunks:
+            assert c.workspace_bytes <= cap, (case, shapes, cap)
+            _check_chunk(lib, c)
+            if c.aol:
+                aol = c.aol_descs(1 << 20)
+                rc = lib.muon_amd_validate_aol(_lib.host_ptr(aol), c.nmat, _lib.host_ptr(c.aol_row_prefix),
+                                               _lib.host_ptr(c.aol_seg_prefix))
+                assert rc == 0, lib.muon_amd_last_error()
 
 
 def test_validation_catches_a_bad_table():
