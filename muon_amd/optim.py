@@ -99,7 +99,7 @@ class _MuonBase(torch.optim.Optimizer):
         stride = (p.numel() // count) * p.element_size()
         for k in range(count):
             eng.early_momentum(first + k, g.data_ptr() + k * stride, m.data_ptr() + k * stride,
-                               beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad)
+                               beta=float(group["momentum"]), nesterov=NESTEROV, mutate_grad=self._mutate_grad)
 
     def __getstate__(self):
         # torch's Optimizer pickles defaults/state/param_groups only; the keyword-only options of
@@ -197,9 +197,11 @@ class _MuonBase(torch.optim.Optimizer):
             self._muon_engines[key] = eng
             self._graphs.pop(device, None)        # a recorded step refers to the engine that was replaced
         n = len(shapes)
+        # float(): schedulers and checkpoints may leave 0-dim tensors in the group (the reference's
+        # tensor arithmetic takes them as they are)
         eng.prepare(grads, moms, ptrs, [0] * n, scales, dtypes,
-                    beta=group["momentum"], nesterov=NESTEROV, mutate_grad=self._mutate_grad,
-                    eps=1e-7, lr=group["lr"], weight_decay=group["weight_decay"])
+                    beta=float(group["momentum"]), nesterov=NESTEROV, mutate_grad=self._mutate_grad,
+                    eps=1e-7, lr=float(group["lr"]), weight_decay=float(group["weight_decay"]))
         self._pending.append(eng)
         self._writebacks += writebacks
         self._keepalive.append(keep)
@@ -235,8 +237,9 @@ class _MuonBase(torch.optim.Optimizer):
             eng.prepare([t[0].data_ptr() for _, t in items], [t[1].data_ptr() for _, t in items],
                         [t[2].data_ptr() for _, t in items], [t[3].data_ptr() for _, t in items],
                         [0] * len(items),
-                        lr=group["lr"], weight_decay=group["weight_decay"], betas=group["betas"],
-                        eps=group["eps"], step=step, dtypes=[_src_dtype(p) for p, _ in items])
+                        lr=float(group["lr"]), weight_decay=float(group["weight_decay"]),
+                        betas=(float(group["betas"][0]), float(group["betas"][1])),
+                        eps=float(group["eps"]), step=step, dtypes=[_src_dtype(p) for p, _ in items])
             self._pending.append(eng)
             self._keepalive.append(items)
         self._writebacks += writebacks

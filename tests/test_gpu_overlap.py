@@ -133,3 +133,33 @@ def test_overlap_refuses_a_second_backward_and_a_replaced_gradient(M):
     opt.step()
     torch.cuda.synchronize()
     assert all(torch.isfinite(p).all() for p in params)
+
+
+def test_tensor_hyper_parameters_and_side_streams_change_nothing(M):
+    """0-dim tensors as lr / weight decay / momentum / betas (schedulers and checkpoints leave them
+    in the groups) give the bits of the same values as floats, and so do steps issued under
+    torch.cuda.stream(...) of alternating streams with the usual event ordering between them."""
+    pa, pb = _params(80), _params(80)
+    ga, gb = (torch.nn.Parameter(torch.ones(33, device="cuda")) for _ in range(2))
+    plain = _make(M, pa, ga)
+    t64 = lambda v: torch.tensor(v, dtype=torch.float64)       # the same double as the python float
+    other = M.SingleDeviceMuonWithAuxAdam(
+        [dict(params=pb, use_muon=True, lr=t64(0.02), weight_decay=t64(0.01).cuda(), momentum=t64(0.95)),
+         dict(params=[gb], use_muon=False, lr=t64(3e-4), weight_decay=0.0, betas=(t64(0.9), t64(0.95)),
+              eps=t64(1e-10))])
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    main = torch.cuda.current_stream()
+    for step in range(4):
+        xs = _inputs(pa, 400 + step)
+        for opt, params, gain in ((plain, pa, ga), (other, pb, gb)):
+            opt.zero_grad(set_to_none=True)
+            (_loss(params, xs) + (gain * gain).sum()).backward()
+        plain.step()
+        s = streams[step % 2]
+        s.wait_stream(main)
+        with torch.cuda.stream(s):
+            other.step()
+        main.wait_stream(s)
+        torch.cuda.synchronize()
+        for a, b in zip(pa + [ga], pb + [gb]):
+            assert torch.equal(a.detach(), b.detach()), (step, tuple(a.shape))
