@@ -163,3 +163,39 @@ def test_tensor_hyper_parameters_and_side_streams_change_nothing(M):
         torch.cuda.synchronize()
         for a, b in zip(pa + [ga], pb + [gb]):
             assert torch.equal(a.detach(), b.detach()), (step, tuple(a.shape))
+
+
+def test_usual_training_loop_companions(M):
+    """A learning-rate scheduler, gradient clipping and a gradient scaler around the optimizer, as a
+    training script has them: the scheduler's `initial_lr` key in the groups, its wrapped step(),
+    clipped (in place) gradients and the scaler's unscale / conditional step all go through, and
+    the parameters follow the oracle optimizer driven the same way on the CPU."""
+    gpu = _params(81)
+    cpu = [torch.nn.Parameter(p.detach().cpu().clone()) for p in gpu]
+    og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01)
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01)
+    schedule = lambda step: 1.0 / (1 + step)
+    sg = torch.optim.lr_scheduler.LambdaLR(og, schedule)
+    sc = torch.optim.lr_scheduler.LambdaLR(oc, schedule)
+    scaler = torch.amp.GradScaler("cuda", init_scale=1024.0)          # a power of two: unscaling is exact
+    for step in range(3):
+        xs = _inputs(gpu, 500 + step)
+        og.zero_grad(set_to_none=True)
+        oc.zero_grad(set_to_none=True)
+        scaler.scale(_loss(gpu, xs)).backward()
+        _loss(cpu, xs).backward()
+        scaler.unscale_(og)
+        torch.nn.utils.clip_grad_norm_(gpu, 0.05)
+        torch.nn.utils.clip_grad_norm_(cpu, 0.05)
+        scaler.step(og)
+        scaler.update()
+        oc.step()
+        sg.step()
+        sc.step()
+        assert og.param_groups[0]["lr"] == oc.param_groups[0]["lr"] == 0.02 * schedule(step + 1)
+        for pc, pg in zip(cpu, gpu):
+            # (the gradients themselves come from two matmul implementations here, and lr / |p| is large
+            # for the small matrices: 2e-3 below 256 rows or columns, as for the conv-sized shapes elsewhere)
+            small = pc.ndim != 2 or min(pc.shape) < 256
+            tol = (2e-3 if small else 1e-3) * (1.5 if pc.ndim != 2 else 1.0) * (step + 1) ** 0.5
+            assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= tol, (step, tuple(pc.shape))
