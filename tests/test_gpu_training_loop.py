@@ -1,8 +1,14 @@
-"""overlap_backward=True on the GPU: post-accumulate-grad hooks run a matrix's first Muon stage
-(muon.py:9-10 and the cast of muon.py:277) on a side stream while autograd is still producing
-the other gradients, and step() skips that stage for those matrices.  The result must be the
-bits of the plain step, the step itself must match the oracle, and the two misuse cases the
-option cannot support must raise instead of corrupting the momentum buffers.
+"""What a training loop does around the optimizer, on the GPU, with gradients that a real autograd
+backward produces.
+
+overlap_backward=True: post-accumulate-grad hooks run a matrix's first Muon stage (muon.py:9-10 and
+the cast of muon.py:277) on a side stream while autograd is still producing the other gradients,
+and step() skips that stage for those matrices.  The result must be the bits of the plain step,
+the step itself must match the oracle, and the two misuse cases the option cannot support must
+raise instead of corrupting the momentum buffers.
+
+Also: 0-dim tensors as hyper-parameters, steps issued on side streams, and a scheduler, gradient
+clipping and a gradient scaler wrapped around the optimizer.
 """
 import pytest
 import torch
