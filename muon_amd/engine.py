@@ -66,8 +66,10 @@ class _ChunkRuntime:
             jobs = (chunk.syrk_jobs if ph == _plan.PH_SYRK else
                     chunk.sym_jobs if ph == _plan.PH_POLY else
                     chunk.poly_full_jobs if ph == _plan.PH_POLY_FULL else chunk.full_jobs)
+            full = ph in (_plan.PH_UPD_EVEN, _plan.PH_UPD_ODD, _plan.PH_UPD_LAST)
             _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(gemm[ph]), chunk.nmat,
-                                                  _lib.host_ptr(jobs), len(jobs), chunk.tile_class,
+                                                  _lib.host_ptr(jobs), len(jobs),
+                                                  chunk.update_class if full else chunk.tile_class,
                                                   chunk.split_slots if ph == _plan.PH_SYRK else 0),
                        "validate_gemm")
         self.mat_template = chunk.mat_descs(base)
@@ -226,8 +228,9 @@ class _ChunkRuntime:
         def gemm(name, ph, it, jobs_ptr, njobs, work, extra_flags=0):
             al, be, ga = c.phase_scalars(ph, it)
             split = ph == _plan.PH_SYRK
+            tile_class = c.update_class if jobs_ptr == self.full_jobs_ptr else c.tile_class
             _launch(name, work, lambda: _lib.check(lib.muon_amd_ns_gemm(
-                self.gemm_ptr[ph], jobs_ptr, njobs, c.tile_class, al, be, ga, flags | extra_flags,
+                self.gemm_ptr[ph], jobs_ptr, njobs, tile_class, al, be, ga, flags | extra_flags,
                 self.split_partials_ptr if split else None, self.split_counters_ptr if split else None, s),
                 "ns_gemm"))
 
@@ -258,7 +261,7 @@ class _ChunkRuntime:
                 # the last update product takes the parameter step in its epilogue (muon.py:14, 98-99)
                 al, be, _ = c.phase_scalars(_plan.PH_UPD_LAST, it)
                 _launch("ns_gemm/update_apply", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm_apply(
-                    self.gemm_ptr[_plan.PH_UPD_LAST], self.full_jobs_ptr, len(c.full_jobs), c.tile_class, al, be,
+                    self.gemm_ptr[_plan.PH_UPD_LAST], self.full_jobs_ptr, len(c.full_jobs), c.update_class, al, be,
                     flags, mats, lr, wd_factor, sc_apply, s), "ns_gemm_apply"))
                 return
             ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)

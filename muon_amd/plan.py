@@ -35,6 +35,7 @@ if os.environ.get("MUON_AMD_SUPER"):     # measurement knob: "rows,cols" of the 
 EW_BLOCK_ELEMS = 8192                   # must match muon_amd_elementwise_block_elems()
 NT_TILE = 128                           # must match muon_amd_normalize_tile()
 N_XCD = 8                               # workgroups are dealt round-robin to the 8 XCDs
+RESIDENT_BIG_TILE_WORKGROUPS = 256      # one 256 x 256 workgroup per CU of an MI355X
 # Workspace rows may be made this many elements longer than the padded width (a knob for
 # measurements: on MI355X a power-of-two row pitch measured no slower than a padded one).
 LD_PAD = int(os.environ.get("MUON_AMD_LD_PAD", "0"))
@@ -117,6 +118,26 @@ def matrix_workspace_bytes(rows: int, cols: int, unit: int) -> int:
     mp, np_ = _round_up(m, unit), _round_up(n, unit)
     return (_round_up(mp * (np_ + LD_PAD) * 2, _ALIGN) + 2 * _round_up(np_ * (mp + LD_PAD) * 2, _ALIGN) +
             3 * _round_up(mp * (mp + LD_PAD) * 2, _ALIGN))
+
+
+UPDATE_CLASS = os.environ.get("MUON_AMD_UPDATE_CLASS", "auto")      # measurement knob: "0", "1" or "auto"
+
+
+def update_class_for(tile_class: int, layouts) -> int:
+    """Tile class of the update products X' = a X + B X of a chunk.  They have m x n tiles to
+    spread over the GPU where the symmetric products have only m x m / 2, so a chunk of the
+    128 x 128 class can afford 256 x 256 tiles for them (half the operand traffic per flop, a
+    quarter of the tiles) when its padded sizes are all multiples of 256 and the larger tiles
+    still give every CU one: measured on the 48 matrices of GPT-2-124M, 4 % off the update
+    launches.  Which tiles compute an element does not change its bits."""
+    if tile_class != 0 or UPDATE_CLASS == "0":
+        return tile_class
+    if any(lay.mp % 256 or lay.np_ % 256 for lay in layouts):
+        return tile_class
+    big_tiles = sum((lay.mp // 256) * (lay.np_ // 256) for lay in layouts)
+    if UPDATE_CLASS == "auto" and big_tiles < RESIDENT_BIG_TILE_WORKGROUPS:
+        return tile_class
+    return 1
 
 
 def matrix_scratch_bytes(rows: int, cols: int, tile_class: int, aol: bool) -> int:
@@ -232,7 +253,10 @@ class ChunkPlan:
         self.split_slots = 0
         self.syrk_jobs = self._jobs(sym=True, reduce_over_n=True)
         self.sym_jobs = self._jobs(sym=True, reduce_over_n=False)
-        self.full_jobs = self._jobs(sym=False, reduce_over_n=False)
+        # The update products may run in the 256 x 256 class where the chunk as a whole is in the
+        # 128 x 128 class (see update_class_for).
+        self.update_class = update_class_for(tile_class, self.layouts)
+        self.full_jobs = self._jobs(sym=False, reduce_over_n=False, tile_class=self.update_class)
         # every tile of the m x m polynomial (no mirrored store): the first iteration of "aol4_rows",
         # whose Gram matrix is not symmetric after the row-only rescaling
         self.poly_full_jobs = self._jobs(sym=False, reduce_over_n=False, square=True) if variant == "aol4_rows" else None
@@ -243,10 +267,11 @@ class ChunkPlan:
         self.workspace_bytes = off
 
     # ---- tile job lists -----------------------------------------------------------------
-    def _jobs(self, sym: bool, reduce_over_n: bool, square: bool = False) -> np.ndarray:
-        TR, TC = self.tile_rows, self.tile_cols
+    def _jobs(self, sym: bool, reduce_over_n: bool, square: bool = False, tile_class: int | None = None) -> np.ndarray:
+        tile_class = self.tile_class if tile_class is None else tile_class
+        TR, TC = TILE_DIMS[tile_class]
         ratio = TR // TC
-        si, sj = SUPER_DIMS[self.tile_class]
+        si, sj = SUPER_DIMS[tile_class]
         parts = []
         for k, lay in enumerate(self.layouts):
             mt = lay.mp // TR

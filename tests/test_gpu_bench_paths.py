@@ -211,3 +211,37 @@ def test_workgroups_that_walk_several_jobs_keep_every_path_right(M):
     og.step()
     for pc, pg in zip(cpu, gpu):
         assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= TOL_PARAM, tuple(pc.shape)
+
+
+def test_large_tile_update_products_give_the_same_bits(M, monkeypatch):
+    """A chunk of the 128 x 128 class with enough work runs its update products in 256 x 256 tiles.
+    The choice of tiles must not change a bit: the same step with the choice switched off."""
+    from muon_amd import plan
+    shapes = [(768, 3072)] * 8 + [(3072, 768)] * 6 + [(768, 768)] * 4 + [(256, 2304)] * 3
+    torch.manual_seed(4242)
+    base = [torch.randn(*s) * 0.02 for s in shapes]
+    grads = [[torch.randn(*s) * 1e-3 for s in shapes] for _ in range(2)]
+    results = {}
+    for mode in ("auto", "0"):
+        monkeypatch.setattr(plan, "UPDATE_CLASS", mode)
+        params = [torch.nn.Parameter(b.clone().cuda()) for b in base]
+        opt = M.SingleDeviceMuon(params, lr=0.02, weight_decay=0.01)
+        for g in grads:
+            for p, gi in zip(params, g):
+                p.grad = gi.clone().cuda()
+            opt.step()
+        torch.cuda.synchronize()
+        (eng,) = opt._muon_engines.values()
+        assert [c.update_class for c in eng.chunks] == ([1] if mode == "auto" else [0])
+        results[mode] = [p.detach().clone() for p in params]
+    for a, b, s in zip(results["auto"], results["0"], shapes):
+        assert torch.equal(a, b), s
+    # and the step is the oracle's
+    cpu = [torch.nn.Parameter(b.clone()) for b in base]
+    oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01)
+    for g in grads:
+        for p, gi in zip(cpu, g):
+            p.grad = gi.clone()
+        oc.step()
+    for pc, pg in zip(cpu, results["auto"]):
+        assert O.rel_fro(pg.cpu(), pc.detach()) <= 1e-3 * 2 ** 0.5, tuple(pc.shape)

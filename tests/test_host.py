@@ -65,10 +65,13 @@ def _check_chunk(lib, c):
     g = c.gemm_descs(1 << 20)
     for ph in range(5):
         jobs = c.syrk_jobs if ph == plan.PH_SYRK else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
-        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), c.tile_class,
+        tile_class = c.update_class if jobs is c.full_jobs else c.tile_class     # the update products may use larger tiles
+        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), tile_class,
                                         c.split_slots if ph == plan.PH_SYRK else 0)
         assert rc == 0, lib.muon_amd_last_error()
+    assert c.update_class in (c.tile_class, 1)
     TR, TC = c.tile_rows, c.tile_cols
+    UR, UC = plan.TILE_DIMS[c.update_class]
     for k, l in enumerate(c.layouts):
         mt, nt, ratio = l.mp // TR, l.np_ // TC, TR // TC
         sj = c.sym_jobs[c.sym_jobs["desc"] == k]
@@ -83,8 +86,9 @@ def _check_chunk(lib, c):
                 cover[j0 // TC, i0 // TC:(i0 + TR) // TC] += 1
         assert (cover == 1).all()
         fj = c.full_jobs[c.full_jobs["desc"] == k]
-        got = sorted(zip((fj["i0"] // TR).tolist(), (fj["j0"] // TC).tolist()))
-        assert got == [(i, j) for i in range(mt) for j in range(nt)]
+        got = sorted(zip((fj["i0"] // UR).tolist(), (fj["j0"] // UC).tolist()))
+        assert got == [(i, j) for i in range(l.mp // UR) for j in range(l.np_ // UC)]
+        assert np.all(fj["i0"] % UR == 0) and np.all(fj["j0"] % UC == 0)
         assert l.mp % T == 0 and l.np_ % T == 0 and l.mp >= l.m and l.np_ >= l.n
         assert l.wide == (l.rows <= l.cols)
     # workspace regions do not overlap and stay inside the chunk's workspace
@@ -412,3 +416,15 @@ def test_overlap_backward_option_installs_hooks_and_survives_copies():
     assert all(p._post_accumulate_grad_hooks for g in dup.param_groups if g["use_muon"] for p in g["params"])
     plain = M.SingleDeviceMuon([torch.nn.Parameter(torch.randn(4, 4))])
     assert not plain._overlap_backward and plain._hook_handles == []
+
+
+def test_update_products_take_large_tiles_only_where_they_fill_the_gpu():
+    gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    (c,) = plan.plan_chunks(gpt2, 5, True, 16 << 30)
+    assert c.tile_class == 0 and c.update_class == 1 and len(c.full_jobs) == 12 * (3 * 9 + 3 * 3 + 3 * 12 + 3 * 12)
+    (c,) = plan.plan_chunks([(768, 3072)], 5, True, 16 << 30)            # 36 large tiles: too few for 256 CUs
+    assert c.tile_class == 0 and c.update_class == 0
+    (c,) = plan.plan_chunks([(768, 3072)] * 16 + [(640, 1280)], 5, True, 16 << 30)      # 640 is not a multiple of 256
+    assert c.update_class == 0
+    (c,) = plan.plan_chunks([(4096, 4096)] * 2, 5, True, 16 << 30)
+    assert c.tile_class == 1 and c.update_class == 1
