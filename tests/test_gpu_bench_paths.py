@@ -245,3 +245,32 @@ def test_large_tile_update_products_give_the_same_bits(M, monkeypatch):
         oc.step()
     for pc, pg in zip(cpu, results["auto"]):
         assert O.rel_fro(pg.cpu(), pc.detach()) <= 1e-3 * 2 ** 0.5, tuple(pc.shape)
+
+
+def test_a_hundred_steps_stay_deterministic(M):
+    """100 consecutive steps on a list with both tile classes, a split reduction and an Adam group:
+    an optimizer that replays its recorded graph and an eager one stay bit for bit together, and two
+    eager runs from the same state give the same bits (no launch leaves anything behind for the
+    next one: split counters, workspace reuse across chunks, scalars read from device memory)."""
+    shapes = [(768, 1024), (1024, 1280), (128, 8192), (300, 200), (16, 8, 3, 3)]
+    torch.manual_seed(9090)
+    base = [torch.randn(*s) * 0.02 for s in shapes]
+    grads = [[torch.randn(*s) * 1e-3 for s in shapes] + [torch.randn(77) * 1e-3] for _ in range(4)]
+    finals = []
+    for use_graph, cap in ((False, None), (True, None), (False, 6 << 20)):
+        params = [torch.nn.Parameter(b.clone().cuda()) for b in base]
+        gain = torch.nn.Parameter(torch.ones(77, device="cuda"))
+        opt = M.SingleDeviceMuonWithAuxAdam(
+            [dict(params=params, use_muon=True, lr=0.01, weight_decay=0.01),
+             dict(params=[gain], use_muon=False, lr=1e-3, weight_decay=0.0)], use_graph=use_graph, workspace_bytes=cap)
+        for step in range(100):
+            for p, g in zip(params + [gain], grads[step % 4]):
+                p.grad = g.clone().cuda()
+            opt.step()
+        torch.cuda.synchronize()
+        assert all(torch.isfinite(p).all() for p in params + [gain])
+        finals.append([p.detach().clone() for p in params + [gain]] +
+                      [opt.state[p]["momentum_buffer"].clone() for p in params])
+    for other in finals[1:]:
+        for a, b in zip(finals[0], other):
+            assert torch.equal(a, b)
