@@ -66,6 +66,29 @@ def f_dense(m, n, steps=5):
     return steps * (4 * m * m * n + 2 * m ** 3)
 
 
+def workload_bounds(name):
+    """Lower bounds of one optimizer step of a workload on an MI355X.
+    mfma_ms: the symmetric-minimum Newton-Schulz flops at the dense bf16 peak.
+    hbm_elementwise_ms: 24 B per Muon element + 28 B per Adam element at the HBM peak.
+    hbm_ns_ms: the Newton-Schulz intermediates through HBM once per product, 5 * (6 m n + 8 m^2) bytes
+    per matrix (X read twice and written once, A and B written and read once, bf16): what bounds the
+    iteration of matrices too short (m < ~640) for their products to be MFMA-bound."""
+    muon, adam, _, _, _ = workload_shapes(name)
+    fs = ns_bytes = n_m = n_a = 0
+    for shape, count in muon:
+        r, c = mat2d(shape)
+        m, n = min(r, c), max(r, c)
+        fs += count * f_sym(m, n)
+        ns_bytes += count * 5 * (6 * m * n + 8 * m * m)
+        n_m += count * r * c
+    for shape, count in adam:
+        r, c = mat2d(shape)
+        n_a += count * r * c
+    ew_bytes = 24 * n_m + 28 * n_a
+    return dict(mfma_ms=fs / (PEAK_BF16_TFLOPS * 1e9), hbm_elementwise_ms=ew_bytes / (PEAK_HBM_GBS * 1e6),
+                hbm_ns_ms=ns_bytes / (PEAK_HBM_GBS * 1e6), ns_bytes=ns_bytes, elementwise_bytes=ew_bytes)
+
+
 def mat2d(shape):
     rows = shape[0]
     cols = 1
@@ -86,11 +109,19 @@ def correctness_gates(name):
 
     torch.set_num_threads(host_threads())
     res, failed = {}, []
+    res["effective_bounds"], res["parity_unpinned"] = {}, []
 
-    def gate(key, value, bound):
+    def gate(key, value, bound, nominal=None):
+        """`nominal`: the bound the contract states, when `bound` is a widened one.  A gate that
+        passes only through the widening is listed under "parity_unpinned" instead of counting as
+        a plain pass."""
         res[key] = round(float(value), 6)
+        res["effective_bounds"][key] = round(float(bound), 6)
         if not value <= bound:
             failed.append(f"{key} = {value:.3e} > {bound:.3e}")
+        elif nominal is not None and not value <= nominal:
+            res["parity_unpinned"].append(f"{key}: {float(value):.3e} is above the stated {nominal:.0e}, "
+                                          f"within the widened {float(bound):.3e}")
 
     def ns_gates(tag, g2):
         """Newton-Schulz output for the 2-D input g2 (CPU tensor).  The oracle's bf16 tensor
@@ -107,10 +138,10 @@ def correctness_gates(name):
         spread = O.rel_fro(ref16_gpu, ref16)
         res[f"ns_bf16_oracle_cpu_vs_gpu_evaluation_{tag}"] = round(float(spread), 6)
         gate(f"ns_vs_bf16_gpu_evaluated_{tag}", O.rel_fro(got, ref16_gpu), TOL_NS_BF16)
-        gate(f"ns_vs_bf16_{tag}", O.rel_fro(got, ref16), max(TOL_NS_BF16, spread + 5e-3))
+        gate(f"ns_vs_bf16_{tag}", O.rel_fro(got, ref16), max(TOL_NS_BF16, spread + 5e-3), TOL_NS_BF16)
         # where the reference's own bf16 result is further than 3e-2 from fp32 (small conv
         # shapes), the kernel that follows its rounding sequence inherits that distance
-        gate(f"ns_vs_fp32_{tag}", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3))
+        gate(f"ns_vs_fp32_{tag}", O.rel_fro(got, ref32), max(TOL_NS_FP32, O.rel_fro(ref16, ref32) + 5e-3), TOL_NS_FP32)
 
     torch.manual_seed(97)
     if name == "ns32":
@@ -128,7 +159,7 @@ def correctness_gates(name):
             muon_amd.SingleDeviceMuon([p_g], lr=0.02, weight_decay=0.01, momentum=0.95).step()
             # a tiny filter's update is several per cent of |p|, so bf16 Newton-Schulz noise weighs more there
             gate(f"param_after_step_{tag}", O.rel_fro(p_g.detach().cpu(), p_c.detach()),
-                 TOL_PARAM if min(mat2d(shape)) >= 128 else 3e-3)
+                 TOL_PARAM if min(mat2d(shape)) >= 128 else 3e-3, TOL_PARAM)
         for shape, _ in adam:
             sl = (min(shape[0], 4096),) + tuple(shape[1:])
             tag = "x".join(str(v) for v in sl)
@@ -384,6 +415,25 @@ def secondary(name, gates):
         out["ms_per_step"] = round(plain["ms_per_step"], 3)
         g = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], use_graph=True)
         out["ms_per_step_graph_replay"] = round(g["ms_per_step"], 3)
+    if name != "ns32":
+        b = workload_bounds(name)
+        if name == "conv":
+            # every matrix is short: the whole step is HBM / latency bound
+            bound_ms = b["hbm_ns_ms"] + b["hbm_elementwise_ms"]
+            out["hbm_roofline"] = {
+                "bound": "hbm", "algorithmic_bytes": b["ns_bytes"] + b["elementwise_bytes"],
+                "what": "5*(6mn+8m^2) B per matrix + 24 B per Muon element + 28 B per Adam element",
+                "achieved_gbs": round((b["ns_bytes"] + b["elementwise_bytes"]) / out["ms_per_step"] / 1e6, 1),
+                "peak_gbs": PEAK_HBM_GBS}
+            out["hbm_frac"] = round(bound_ms / out["ms_per_step"], 4)
+        else:
+            # MFMA-bound products + HBM-bound elementwise kernels, one after the other
+            bound_ms = b["mfma_ms"] + b["hbm_elementwise_ms"]
+            out["bound_parts_ms"] = {"mfma": round(b["mfma_ms"], 4), "hbm_elementwise": round(b["hbm_elementwise_ms"], 4)}
+        out["bound_ms"] = round(bound_ms, 4)
+        out["bound_frac"] = round(bound_ms / out["ms_per_step"], 4)
+        r = run_optimizer_workload(name, dsteps, dwarm, seed=SECONDARY_SEEDS[name], realloc_grads=True, launch_events=False)
+        out["ms_per_step_realloc_grads"] = round(r["ms_per_step"], 3)
     if name == "gpt2-124m":
         out["backward_overlap"] = run_backward_overlap(name)
     return out

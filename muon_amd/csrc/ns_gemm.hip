@@ -31,6 +31,7 @@
 
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -897,7 +898,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxDevices = 64;
 struct DeviceState {
-    bool ready = false;
+    std::atomic<bool> ready{false};           // set (release) once the fields below are final
     int num_cus = 0;                          // a persistent launch has num_cus * MINB workgroups at most
     unsigned char* scratch_ptr = nullptr;     // device address of `scratch` on this device
 };
@@ -923,9 +924,13 @@ static int device_setup(const DeviceState** out) {
         set_error("no usable HIP device is current (device index %d)", dev);
         return MUON_AMD_EDEVICE;
     }
-    std::lock_guard<std::mutex> lock(g_devices_mutex);
     DeviceState& st = g_devices[dev];
-    if (!st.ready) {
+    if (st.ready.load(std::memory_order_acquire)) {     // every launch after the first: no lock
+        *out = &st;
+        return MUON_AMD_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_devices_mutex);
+    if (!st.ready.load(std::memory_order_relaxed)) {
         hipDeviceProp_t prop;
         if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
             (void)hipGetLastError();
@@ -949,7 +954,7 @@ static int device_setup(const DeviceState** out) {
         }
         st.scratch_ptr = static_cast<unsigned char*>(ptr);
         st.num_cus = prop.multiProcessorCount;
-        st.ready = true;
+        st.ready.store(true, std::memory_order_release);
     }
     *out = &st;
     return MUON_AMD_OK;

@@ -43,19 +43,44 @@ def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def _upload(arr: np.ndarray, device, into: torch.Tensor | None = None) -> torch.Tensor:
-    """Async host->device copy of a table through pinned staging (no stream or host sync).
-    With `into`, the bytes land in that existing device buffer, whose address launches recorded
-    in a HIP graph keep referring to."""
+def _upload(arr: np.ndarray, device) -> torch.Tensor:
+    """Async host->device copy of a table that is uploaded once, through pinned staging (no stream
+    or host sync)."""
     host = torch.from_numpy(np.ascontiguousarray(arr).view(np.uint8).reshape(-1)).pin_memory()
-    if into is None:
-        return host.to(device, non_blocking=True)
-    into.copy_(host, non_blocking=True)
-    return into
+    return host.to(device, non_blocking=True)
+
+
+class _Staging:
+    """One pinned host buffer for the tables an engine uploads again and again (matrix descriptors
+    after a tensor moved, Adam descriptors, a graph's scalars): the bytes are copied into it and from
+    there to the device asynchronously.  Before the buffer is overwritten the host waits for the
+    copy that last read it, which has normally finished long ago."""
+
+    def __init__(self, device):
+        self.device = device
+        self.host = None
+        self.event = None
+
+    def upload(self, arr: np.ndarray, into: torch.Tensor) -> torch.Tensor:
+        src = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+        n = src.size
+        assert into.numel() == n, (into.numel(), n)
+        if self.host is None or self.host.numel() < n:
+            if self.event is not None:
+                self.event.synchronize()
+            self.host = torch.empty(max(n, 4096), dtype=torch.uint8, pin_memory=True)
+            self.event = torch.cuda.Event()
+        else:
+            self.event.synchronize()
+        self.host[:n].numpy()[:] = src
+        into.copy_(self.host[:n], non_blocking=True)
+        self.event.record(torch.cuda.current_stream(self.device))
+        return into
 
 
 class _ChunkRuntime:
     def __init__(self, chunk: _plan.ChunkPlan, base: int, device):
+        self.staging = _Staging(device)
         lib = _lib.load()
         self.chunk = chunk
         self.device = device
@@ -137,7 +162,9 @@ class _ChunkRuntime:
                                               _lib.host_ptr(self.chunk.block_prefix),
                                               _lib.host_ptr(self.chunk.tile_prefix), self.chunk.tile),
                    "validate_mats")
-        self.mat_dev = _upload(d, self.device, into=self.mat_dev)
+        if self.mat_dev is None:
+            self.mat_dev = torch.empty(d.nbytes, dtype=torch.uint8, device=self.device)
+        self.staging.upload(d, self.mat_dev)
         self.mat_key = key
         self.mat_host = d
         self.src_dtypes = list(src_dtypes)
@@ -156,7 +183,7 @@ class _ChunkRuntime:
                                               _lib.host_ptr(self.chunk.tile_prefix), self.chunk.tile),
                    "validate_mats")
         sz = _lib.MAT_DESC.itemsize
-        _upload(d[k:k + 1], self.device, into=self.mat_dev[k * sz:(k + 1) * sz])
+        self.staging.upload(d[k:k + 1], self.mat_dev[k * sz:(k + 1) * sz])
         g, m, *rest = self.mat_key
         g, m = list(g), list(m)
         g[k], m[k] = grad, momentum
@@ -302,7 +329,7 @@ class MuonGroupEngine:
         self._early_pos = {lay.index: k for k, lay in enumerate(self.chunks[0].layouts)}
         self._early_stream = None
         self._early_events = {}
-        self._early_done = {}         # position -> gradient address the stage consumed
+        self._early_done = {}         # position -> (gradient address, caller's token) the stage consumed
         self._skip = frozenset()
 
     def prepare(self, grads, momenta, params, outs, scales, src_dtypes, *, beta, nesterov, mutate_grad,
@@ -314,7 +341,7 @@ class MuonGroupEngine:
             torch.cuda.current_stream(self.device).wait_stream(self._early_stream)
             layouts = self.chunks[0].layouts
             done, self._early_done = self._early_done, {}
-            for k, used in done.items():
+            for k, (used, _) in done.items():
                 if grads[layouts[k].index] != used:
                     raise _lib.MuonAmdError(
                         f"the gradient of matrix {layouts[k].index} was replaced after its momentum stage ran "
@@ -346,25 +373,48 @@ class MuonGroupEngine:
             rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
                    h["wd_factor"], scalars_ptr=scalars_ptr, momentum_done=self._skip if n == 0 else frozenset())
 
-    def early_momentum(self, i, grad, momentum, *, beta, nesterov, mutate_grad) -> bool:
+    def early_stream(self):
+        """The side stream the early stages run on (default priority; created on first use)."""
+        if self._early_stream is None:
+            self._early_stream = torch.cuda.Stream(self.device)
+        return self._early_stream
+
+    def early_eligible(self, i) -> bool:
+        """Whether `early_momentum` would act on matrix `i`: it is in the first chunk and a step has run."""
+        return i in self._early_pos and self.runtimes[0].mat_key is not None
+
+    def early_pending(self, i):
+        """(gradient address, token) the pending early stage of matrix `i` consumed, or None."""
+        k = self._early_pos.get(i)
+        return None if k is None else self._early_done.get(k)
+
+    def early_discard(self, i) -> None:
+        """Forget the pending early stage of matrix `i`: the next step runs its momentum stage itself.
+        The caller has put the momentum buffer back to what it was before that stage."""
+        k = self._early_pos.get(i)
+        if k is not None:
+            self._early_done.pop(k, None)
+
+    def early_momentum(self, i, grad, momentum, *, beta, nesterov, mutate_grad, token=None, redo=False) -> bool:
         """Run the first stage of matrix `i` (position in `shapes`) -- momentum, Nesterov blend,
         bf16 cast, sums of squares -- now, on a side stream that first waits for everything enqueued
         so far on the current stream (the work that produced the gradient), instead of inside the
         step.  The next `prepare` joins the side stream, and that step's `enqueue` leaves the matrix
         out of its momentum launch.  Meant to be called from a hook that fires during backward once
-        the gradient at address `grad` is complete.  Returns False, having done nothing, for a
-        matrix outside the first chunk or an engine that has not run a step yet."""
+        the gradient at address `grad` is complete; `token` is kept beside the address for the
+        caller (`early_pending`).  A second stage for a matrix before a step raises unless `redo`
+        says that the caller has put the momentum buffer back (on the side stream) to what it was
+        before the first one.  Returns False, having done nothing, for a matrix outside the first
+        chunk or an engine that has not run a step yet."""
         k = self._early_pos.get(i)
         rt = self.runtimes[0]
         if k is None or rt.mat_key is None:
             return False
-        if k in self._early_done:
+        if k in self._early_done and not redo:
             raise _lib.MuonAmdError(
-                f"matrix {i}: a second gradient arrived before step() (overlap with backward supports one "
-                "backward pass per step; the momentum buffer has already taken the first gradient)")
-        if self._early_stream is None:
-            self._early_stream = torch.cuda.Stream(self.device)
-        side = self._early_stream
+                f"matrix {i}: a second gradient arrived before step() (the momentum buffer has already "
+                "taken the first one; restore it and pass redo=True)")
+        side = self.early_stream()
         ev = self._early_events.get(k)
         if ev is None:
             ev = self._early_events[k] = torch.cuda.Event()
@@ -378,7 +428,7 @@ class MuonGroupEngine:
                 rt.momentum_of(k, 1 - beta, beta, nesterov, mutate_grad)
         else:       # the common case, kept cheap: this runs once per matrix inside backward
             rt.momentum_of(k, 1 - beta, beta, nesterov, mutate_grad, stream=side.cuda_stream)
-        self._early_done[k] = grad
+        self._early_done[k] = (grad, token)
         return True
 
     def run(self, grads, momenta, params, outs, scales, src_dtypes, **hyper):
@@ -400,6 +450,7 @@ class AdamGroupEngine:
         self.prefix_dev = _upload(self.prefix, self.device)
         # one buffer for the descriptors, rewritten in place: recorded launches keep its address
         self.desc_dev = torch.empty(len(self.numels) * _lib.ADAM_DESC.itemsize, dtype=torch.uint8, device=self.device)
+        self.staging = _Staging(self.device)
         self.key = None
         self._hyper = None
 
@@ -416,7 +467,7 @@ class AdamGroupEngine:
             d["update"] = updates
             d["numel"] = self.numels
             d["dtype"] = dtypes
-            _upload(d, self.device, into=self.desc_dev)
+            self.staging.upload(d, self.desc_dev)
             self.key = key
             self.nbytes = sum(n * (14 if t == _lib.SRC_BF16 else 28) for n, t in zip(self.numels, dtypes))
         # python doubles, as muon.py:105-108 and 257
@@ -454,6 +505,7 @@ class StepGraph:
         self.graph = None
         self.key = None
         self.scalars = None
+        self.staging = _Staging(self.device)
         self.replays = 0
 
     def run(self, engines):
@@ -466,8 +518,7 @@ class StepGraph:
         if self.scalars is None or self.scalars.numel() < len(host):
             self.scalars = torch.zeros(max(len(host), 16), dtype=torch.float32, device=self.device)
             self.graph = None                                    # recorded launches hold the old address
-        _upload(np.asarray(host, dtype=np.float32), self.device,
-                into=self.scalars.view(torch.uint8)[: 4 * len(host)])
+        self.staging.upload(np.asarray(host, dtype=np.float32), self.scalars.view(torch.uint8)[: 4 * len(host)])
         key = tuple(e.structure_key() for e in engines)
         if self.graph is None or key != self.key:
             graph = torch.cuda.CUDAGraph()

@@ -32,7 +32,8 @@ class _MuonBase(torch.optim.Optimizer):
                       overlap_backward=False):
         self._use_graph = bool(use_graph)
         self._overlap_backward = bool(overlap_backward)
-        self._early_params = {}       # Muon parameter -> (engine, first matrix, matrices, group), set by each step
+        self._early_params = {}       # Muon parameter -> (engine, first matrix, matrices, group index), set by each step
+        self._early_shadow = {}       # Muon parameter -> copy of its momentum buffer from before a pending early stage
         self._install_overlap_hooks()
         if ns_variant not in ("ns5", "aol4", "aol4_rows"):
             raise ValueError(f"ns_variant must be 'ns5', 'aol4' or 'aol4_rows', got {ns_variant!r}")
@@ -47,6 +48,7 @@ class _MuonBase(torch.optim.Optimizer):
         self._pending = []            # engines prepared by the group loop of the current step, in launch order
         self._writebacks = []         # (destination, contiguous copy) pairs to copy back after the launches
         self._keepalive = []          # temporaries whose addresses the pending launches use
+        self._step_bumps = []         # (Adam state, new step count) written when the launches go out
 
     _RUNTIME_OPTIONS = ("_ns_rounding", "_mutate_grad", "_workspace_bytes", "_ns_variant", "_use_graph",
                         "_overlap_backward")
@@ -84,22 +86,75 @@ class _MuonBase(torch.optim.Optimizer):
     @torch.no_grad()
     def _grad_ready(self, p):
         """Autograd has finished accumulating p.grad (post-accumulate-grad hook).  Once a step has
-        built the group's engine, enqueue the matrix's momentum stage on the engine's side stream;
-        step() then skips it.  Anything out of the ordinary (no engine yet, strided tensors, a
-        gradient of another dtype) is left to step()."""
+        built the group's engine, enqueue the momentum stage of the parameter's matrices on the
+        engine's side stream; step() then skips it.  The momentum buffer is copied aside first, so
+        that the stage can be taken back: when a second gradient arrives before step() (gradients
+        accumulated over micro-batches, or a step that was skipped) the buffer is restored and the
+        stage runs again on the gradient as it is now, and step() takes the stage back when the
+        gradient was touched after it ran (`_early_settle`).  Anything out of the ordinary (no
+        engine yet, strided tensors, a gradient of another dtype, mutate_grad) is left to step()."""
         info = self._early_params.get(p)
-        if info is None:
+        if info is None or self._mutate_grad:     # a stage that overwrote the gradient could not run again
             return
-        eng, first, count, group = info
+        eng, first, count, gi = info
+        if gi >= len(self.param_groups):
+            return
+        group = self.param_groups[gi]             # looked up now: load_state_dict replaces the group dicts
         g, m = p.grad, self.state[p].get("momentum_buffer")
         if (g is None or m is None or g.is_sparse or g.dtype != p.dtype or m.dtype != p.dtype or
                 m.shape != p.shape or g.device != p.device or m.device != p.device or
                 not (g.is_contiguous() and m.is_contiguous() and p.is_contiguous())):
             return
+        if not all(eng.early_eligible(first + k) for k in range(count)):
+            return
+        pending = eng.early_pending(first)
+        if pending is not None and pending[1][2] != m.data_ptr():
+            for k in range(count):                # the state tensor was replaced since: nothing to take back
+                eng.early_discard(first + k)
+            pending = None
+        shadow = self._early_shadow.get(p)
+        if pending is None and (shadow is None or shadow.shape != m.shape or shadow.dtype != m.dtype or
+                                shadow.device != m.device):
+            shadow = self._early_shadow[p] = torch.empty_like(m)
+        side = eng.early_stream()
+        side.wait_stream(torch.cuda.current_stream(p.device))
+        with torch.cuda.stream(side):
+            if pending is not None:
+                m.copy_(shadow)                   # the buffer as it was before the stage that is discarded
+            else:
+                shadow.copy_(m)
         stride = (p.numel() // count) * p.element_size()
+        # The gradient tensor itself is part of the token: holding it keeps its memory from being
+        # handed out again while the side stream reads it, and lets step() tell this tensor from a
+        # new one that the allocator put at the same address.
+        token = (g, g._version, m.data_ptr())
         for k in range(count):
             eng.early_momentum(first + k, g.data_ptr() + k * stride, m.data_ptr() + k * stride,
-                               beta=float(group["momentum"]), nesterov=NESTEROV, mutate_grad=self._mutate_grad)
+                               beta=float(group["momentum"]), nesterov=NESTEROV, mutate_grad=False,
+                               token=token, redo=pending is not None)
+
+    def _early_settle(self, p, eng, first, g, m, plain):
+        """step() is about to use parameter p as matrices first.. of engine `eng` (None: another
+        engine).  A pending early stage stands if it consumed exactly this gradient (the same tensor
+        object, not written since: torch counts in-place writes in `_version`) into this momentum
+        buffer; otherwise it is taken back: the buffer is restored from the copy made before the
+        stage, and the step runs the stage itself."""
+        info = self._early_params.get(p)
+        if info is None:
+            return
+        old_eng, old_first, count, _ = info
+        pending = old_eng.early_pending(old_first)
+        if pending is None:
+            return
+        addr, (staged_grad, version, m_addr) = pending
+        if (plain and old_eng is eng and old_first == first and g is staged_grad and g.data_ptr() == addr and
+                g._version == version and m.data_ptr() == m_addr):
+            return
+        if m.data_ptr() == m_addr:
+            torch.cuda.current_stream(p.device).wait_stream(old_eng.early_stream())
+            m.copy_(self._early_shadow[p])
+        for k in range(count):
+            old_eng.early_discard(old_first + k)
 
     def __getstate__(self):
         # torch's Optimizer pickles defaults/state/param_groups only; the keyword-only options of
@@ -196,6 +251,10 @@ class _MuonBase(torch.optim.Optimizer):
                                       variant=self._ns_variant)
             self._muon_engines[key] = eng
             self._graphs.pop(device, None)        # a recorded step refers to the engine that was replaced
+        if self._overlap_backward:
+            plain = {id(p): first for p, first, _ in spans}
+            for p in params:
+                self._early_settle(p, eng, plain.get(id(p)), p.grad, self.state[p]["momentum_buffer"], id(p) in plain)
         n = len(shapes)
         # float(): schedulers and checkpoints may leave 0-dim tensors in the group (the reference's
         # tensor arithmetic takes them as they are)
@@ -209,7 +268,7 @@ class _MuonBase(torch.optim.Optimizer):
             for p in params:
                 self._early_params.pop(p, None)
             for p, first, count in spans:
-                self._early_params[p] = (eng, first, count, group)
+                self._early_params[p] = (eng, first, count, gi)
 
     def _adam_group_step(self, gi, group):
         by_step, writebacks = {}, []
@@ -221,12 +280,16 @@ class _MuonBase(torch.optim.Optimizer):
                 state["exp_avg"] = torch.zeros_like(p, memory_format=torch.contiguous_format)
                 state["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.contiguous_format)
                 state["step"] = 0
-            state["step"] += 1                    # muon.py:254
+            # muon.py:254 increments before the update; the new count is written to the state when the
+            # launches go out (_launch_pending), so that a step that raises while a later group is
+            # prepared leaves every counter where it was
+            step_now = int(state["step"]) + 1
+            self._step_bumps.append((state, step_now))
             if p.numel() > 0:
                 item = (self._dense(p, writebacks), self._dense(g, writebacks, written=False),
                         self._dense(self._state_tensor(state, "exp_avg", p), writebacks),
                         self._dense(self._state_tensor(state, "exp_avg_sq", p), writebacks))
-                by_step.setdefault(int(state["step"]), []).append((p, item))
+                by_step.setdefault(step_now, []).append((p, item))
         for step, items in by_step.items():
             device = items[0][0].device
             key = (gi, device, tuple(id(p) for p, _ in items))
@@ -249,6 +312,8 @@ class _MuonBase(torch.optim.Optimizer):
         per device that is replayed every step; then copy back tensors that went through a
         contiguous copy (stream ordered after the launches)."""
         try:
+            for state, step_now in self._step_bumps:
+                state["step"] = step_now
             by_device = {}
             for eng in self._pending:
                 by_device.setdefault(eng.device, []).append(eng)
@@ -265,10 +330,11 @@ class _MuonBase(torch.optim.Optimizer):
             for dst, src in self._writebacks:
                 dst.copy_(src)
         finally:
-            self._pending, self._writebacks, self._keepalive = [], [], []
+            self._pending, self._writebacks, self._keepalive, self._step_bumps = [], [], [], []
 
     def _run_closure(self, closure):
-        self._pending, self._writebacks, self._keepalive = [], [], []     # nothing left over from a step that raised
+        # nothing left over from a step that raised
+        self._pending, self._writebacks, self._keepalive, self._step_bumps = [], [], [], []
         loss = None
         if closure is not None:
             with torch.enable_grad():
@@ -292,11 +358,15 @@ class SingleDeviceMuon(_MuonBase):
     overlap_backward (post-accumulate-grad hooks on the Muon parameters run a matrix's first stage
     -- momentum, Nesterov blend, bf16 cast, sums of squares -- on a side stream as soon as backward
     has produced its gradient, and step() skips it; from the second step on, for the matrices of
-    the first workspace chunk.  It needs exactly one backward pass per step and gradients that
-    nothing touches between backward and step -- no accumulation over micro-batches, no clipping;
-    a second gradient or a replaced gradient tensor raises.  The momentum buffers take the gradient
-    when backward produces it: a step() that is then skipped, as a loss scaler does after an
-    overflow, leaves them updated all the same).
+    the first workspace chunk.  The stage can be taken back: the momentum buffer is copied aside
+    before it runs, a second gradient before step() -- accumulation over micro-batches, or a step
+    that was skipped, as a loss scaler does after an overflow -- restores the buffer and runs the
+    stage again on the gradient as it then is, and step() restores the buffer and runs the stage
+    itself when the gradient was written after the stage (in-place clipping or unscaling: torch's
+    version counter of the gradient tensor tells) or replaced.  What remains: between backward and
+    step() the momentum buffer of a staged parameter holds the not-yet-committed value, and
+    mutate_grad=True switches the early stage off).  Hyper-parameters kept as 0-dim tensors on the
+    GPU are read with float(), which waits for the device once per step and group.
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0, momentum=0.95, *, ns_rounding="reference",

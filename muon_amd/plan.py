@@ -26,6 +26,14 @@ AOL_COEFFS = ((4.0098, -7.0585, 2.4635), (3.4585, -5.5479, 2.5959),
               (2.7573, -3.2939, 1.4254), (2.7215, -3.0494, 1.3169))
 # "aol4": the Gram matrix rescaled on both sides; "aol4_rows": by rows only, as muon.py:785 writes it
 VARIANTS = ("ns5", "aol4", "aol4_rows")
+# The rows-only rescaling (muon.py:785 as written) is refused for matrices with a side shorter than
+# this.  Dividing the rows of A by s while X is divided by sqrt(s) leaves the first polynomial with a
+# matrix that is not the Gram matrix of X; for a short matrix the row sums s_i scatter enough that the
+# iteration stops contracting: in float64, on Gaussian matrices whose row norms vary by +-5 %, the
+# largest singular value of the result reaches 1.4 for 32 x 32, 58 for 28 x 28, 1e3 for 24 x 24 and
+# 1e18 for 6 x 30, and rounding differences are amplified alike (a bf16 evaluation is up to 1.1 in
+# relative Frobenius norm from the float64 one at 18 x 63), so no error bound can be stated below it.
+AOL_ROWS_MIN_SIDE = 32
 AOL_ROWS = 4                            # must match muon_amd_aol_rows_per_block()
 TILE_DIMS = {0: (128, 128), 1: (256, 256)}   # must match muon_amd_gemm_tile_rows/cols()
 # output tiles (rows, cols) of one XCD-resident super-block: as many tiles as an XCD holds workgroups
@@ -411,6 +419,13 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
     buffers and the scratch beside them) stays under `workspace_cap` bytes (a single matrix larger
     than the cap gets a chunk of its own).
     Same-shape matrices are kept together so that their tiles batch into full waves of the GPU."""
+    if variant == "aol4_rows":
+        short = [tuple(sh) for sh in shapes if min(sh) < AOL_ROWS_MIN_SIDE]
+        if short:
+            raise ValueError(
+                f"the rows-only AOL rescaling is not offered for matrices with a side below {AOL_ROWS_MIN_SIDE} "
+                f"(got {short[0][0]} x {short[0][1]}): the iteration does not contract there and amplifies rounding "
+                "differences without bound; use the symmetric rescaling (ns_variant='aol4', rescale='symmetric')")
     order = sorted(range(len(shapes)),
                    key=lambda i: (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]),
                                   -shapes[i][0], i))

@@ -557,7 +557,7 @@ def test_aol4_rows_only_rescaling_matches_its_oracle(M, shape, std):
 
 
 def test_aol4_rows_only_optimizer_step(M):
-    shapes = [(256, 384), (384, 256), (16, 8, 3, 3)]
+    shapes = [(256, 384), (384, 256), (32, 8, 3, 3)]
     cpu, gpu = _clone_params(shapes, 0.02, 1322)
     oc = O.OracleSingleDeviceMuon(cpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns=O.ns_aol4_rows)
     og = M.SingleDeviceMuon(gpu, lr=0.02, weight_decay=0.01, momentum=0.95, ns_variant="aol4_rows")
@@ -567,6 +567,61 @@ def test_aol4_rows_only_optimizer_step(M):
         og.step()
         for pc, pg in zip(cpu, gpu):
             assert O.rel_fro(pg.detach().cpu(), pc.detach()) <= 2e-3, (tuple(pc.shape), step)
+
+
+# Thin matrices (a side of 2 .. 24).  With a handful of singular values the bf16 roundings of the
+# small Gram matrix do not average out: the bf16 oracle itself sits 3e-2 .. 9e-2 (2 x 65: 0.23) from
+# the float64 closed form, and the kernel, which agrees with the bf16 oracle to better than 1e-2,
+# inherits that distance.  So the second bound is the oracle's own distance + 5e-3 where that is larger.
+THIN_SHAPES = [((9, 889), 1e-3), ((1024, 10), 1e-2), ((17, 1605), 5e-2), ((63, 6), 0.3), ((2, 65), 1e-3),
+               ((1136, 24), 0.5), ((7, 767), 1e-3), ((24, 24), 1.0), ((3, 127), 1e-2), ((1797, 4), 0.1)]
+
+
+@pytest.mark.parametrize("shape,std", THIN_SHAPES)
+@pytest.mark.parametrize("uneven", [False, True])
+def test_aol4_on_thin_matrices(M, shape, std, uneven):
+    torch.manual_seed(hash(shape) % 1000 + 7)
+    G = torch.randn(*shape) * std
+    if uneven:
+        G = G * (torch.rand(shape[0], 1) * 3 + 0.05)
+    got = M.zeropower_via_aol4(_dev(G)).float().cpu()
+    ref16 = O.ns_aol4(G).float()
+    closed = O.ns_aol4_closed_form(G.bfloat16().double().numpy())
+    assert O.rel_fro(got, ref16) <= TOL_BF16
+    own = O.rel_fro(ref16.double(), closed)
+    assert O.rel_fro(got.double(), closed) <= max(TOL_FP32, own + 5e-3), own
+
+
+@pytest.mark.parametrize("shape,std", THIN_SHAPES)
+def test_single_rounding_path_on_thin_matrices(M, shape, std):
+    """rounding="fused" (one rounding per stored matrix) against the fp32 oracle on thin matrices: the
+    reference's own bf16 result is up to 0.13 from fp32 there (four singular values), so the bound is
+    3e-2 or the reference's own distance + 5e-3."""
+    torch.manual_seed(hash(shape) % 1000 + 8)
+    G = torch.randn(*shape) * std
+    got = M.zeropower_via_newtonschulz5(_dev(G), 5, rounding="fused").float().cpu()
+    ref32 = O.ns5_fp32(G.bfloat16().float())
+    own = O.rel_fro(O.ns5_bf16(G).float(), ref32)
+    assert O.rel_fro(got, ref32) <= max(TOL_FP32, own + 5e-3), own
+    assert torch.isfinite(got).all()
+
+
+def test_aol4_rows_only_is_refused_for_short_matrices(M):
+    """Below a side of 32 the rows-only map does not contract (sigma_max of its float64 result: 1e3 at
+    24 x 24, 1e18 at 6 x 30) and amplifies rounding differences without bound, so nothing could be
+    compared: it raises, from the functional entry point and from an optimizer step; 32 and above run."""
+    for shape in [(18, 63), (63, 18), (31, 31), (6, 30)]:
+        with pytest.raises(ValueError, match="rows-only"):
+            M.zeropower_via_aol4(torch.randn(*shape, device="cuda"), rescale="rows")
+    p = torch.nn.Parameter(torch.randn(16, 8, 3, 3, device="cuda") * 0.02)
+    p.grad = torch.randn_like(p) * 1e-2
+    with pytest.raises(ValueError, match="rows-only"):
+        M.SingleDeviceMuon([p], ns_variant="aol4_rows").step()
+    for shape in [(32, 100), (40, 63), (63, 40)]:
+        torch.manual_seed(shape[0])
+        G = torch.randn(*shape) * 1e-2 * (1 + 0.1 * (torch.rand(shape[0], 1) - 0.5))
+        got = M.zeropower_via_aol4(_dev(G), rescale="rows").float().cpu()
+        assert O.rel_fro(got, O.ns_aol4_rows(G).float()) <= TOL_BF16, shape
 
 
 def test_aol4_batched_special_inputs_and_optimizer_step(M):

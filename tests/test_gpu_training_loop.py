@@ -4,8 +4,8 @@ backward produces.
 overlap_backward=True: post-accumulate-grad hooks run a matrix's first Muon stage (muon.py:9-10 and
 the cast of muon.py:277) on a side stream while autograd is still producing the other gradients,
 and step() skips that stage for those matrices.  The result must be the bits of the plain step,
-the step itself must match the oracle, and the two misuse cases the option cannot support must
-raise instead of corrupting the momentum buffers.
+the step itself must match the oracle, and a gradient that changes after its early stage ran
+(accumulation, clipping, replacement, a skipped step) must give the plain optimizer's bits too.
 
 Also: 0-dim tensors as hyper-parameters, steps issued on side streams, and a scheduler, gradient
 clipping and a gradient scaler wrapped around the optimizer.
@@ -114,31 +114,71 @@ def test_overlapped_step_matches_the_oracle(M):
     assert len(next(iter(og._muon_engines.values()))._skip) == len(SHAPES) + 2       # the 3-D parameter is three matrices
 
 
-def test_overlap_refuses_a_second_backward_and_a_replaced_gradient(M):
-    from muon_amd._lib import MuonAmdError
+def _drive(M, scenario, overlap):
+    """Six iterations of one training-loop scenario; returns parameters and momentum buffers."""
     params = _params(79)
-    opt = M.SingleDeviceMuon(params, overlap_backward=True)
-    xs = _inputs(params, 300)
-    _loss(params, xs).backward()
-    opt.step()                                   # builds the engine; hooks act from now on
-    opt.zero_grad(set_to_none=True)
-    _loss(params, xs).backward()
-    with pytest.raises(MuonAmdError, match="second gradient"):
-        _loss(params, xs).backward()             # accumulation over micro-batches
-    opt.step()                                   # consumes what the first of the two passes started
-    torch.cuda.synchronize()
-    opt.zero_grad(set_to_none=True)
-    _loss(params, xs).backward()
-    params[0].grad = params[0].grad.clone()      # what a clipping routine that reallocates would do
-    with pytest.raises(MuonAmdError, match="replaced"):
+    opt = M.SingleDeviceMuon(params, lr=0.02, weight_decay=0.01, overlap_backward=overlap)
+    for it in range(6):
+        xs = _inputs(params, 300 + it)
+        opt.zero_grad(set_to_none=(it % 2 == 0))
+        _loss(params, xs).backward()
+        if scenario == "accumulate":             # a second micro-batch accumulates into the same gradients
+            _loss(params, _inputs(params, 900 + it)).backward()
+        elif scenario == "clip_in_place":        # writes the gradients after the hooks consumed them
+            torch.nn.utils.clip_grad_norm_(params, 0.05)
+        elif scenario == "replace":              # what a clipping routine that reallocates does
+            for p in params[::2]:
+                p.grad = p.grad.clone() * 0.5
+        elif scenario == "skip" and it in (2, 3):
+            continue                             # a loss scaler after an overflow: no step() this iteration
+        elif scenario == "skip_none" and it == 2:
+            opt.zero_grad(set_to_none=True)      # skipped, and the next step sees no gradient at all
+            opt.step()
+            continue
         opt.step()
     torch.cuda.synchronize()
-    # the optimizer is usable again afterwards
-    opt.zero_grad(set_to_none=True)
-    _loss(params, xs).backward()
+    staged = len(next(iter(opt._muon_engines.values()))._skip)
+    return [p.detach().clone() for p in params], [opt.state[p]["momentum_buffer"].clone() for p in params], staged
+
+
+@pytest.mark.parametrize("scenario", ["accumulate", "clip_in_place", "replace", "skip", "skip_none"])
+def test_overlap_takes_its_early_stage_back_when_the_gradient_changes(M, scenario):
+    """Gradient accumulation, in-place clipping, replaced gradient tensors and skipped steps under
+    overlap_backward give the bits of the plain optimizer driven the same way: a stage that ran on a
+    gradient that is no longer the one step() sees is undone (the momentum buffer restored) and run
+    again, and a skipped step leaves the momentum untouched as the reference does (muon.py:97 runs
+    inside step() only)."""
+    pa, ma, _ = _drive(M, scenario, overlap=False)
+    pb, mb, staged = _drive(M, scenario, overlap=True)
+    for a, b in zip(pa + ma, pb + mb):
+        assert torch.equal(a, b), (scenario, tuple(a.shape))
+    assert all(torch.isfinite(p).all() for p in pb)
+    if scenario in ("accumulate", "skip", "skip_none"):
+        assert staged == len(SHAPES) + 2         # the last step still found every stage done early
+    elif scenario == "clip_in_place":
+        assert staged == 0                       # every stage was taken back
+    else:
+        assert 0 < staged < len(SHAPES) + 2
+
+
+def test_a_step_that_raises_leaves_the_adam_counters_alone(M):
+    """Groups are prepared before anything is launched; a later group that raises must not leave the
+    Adam step counters of an earlier one advanced (muon.py:254 increments inside the update)."""
+    gain = torch.nn.Parameter(torch.ones(50, device="cuda"))
+    w = torch.nn.Parameter(torch.randn(64, 64, device="cuda") * 0.02)
+    bad = torch.nn.Parameter(torch.randn(64, 64, device="cuda").half())
+    opt = M.SingleDeviceMuonWithAuxAdam([dict(params=[gain], use_muon=False), dict(params=[w], use_muon=True)])
+    for p in (gain, w):
+        p.grad = torch.randn_like(p) * 1e-2
     opt.step()
+    assert opt.state[gain]["step"] == 1
+    opt.add_param_group(dict(params=[bad], use_muon=True, lr=0.02, momentum=0.95, weight_decay=0))
+    bad.grad = torch.randn_like(bad)
+    before = gain.detach().clone()
+    with pytest.raises(NotImplementedError):
+        opt.step()
     torch.cuda.synchronize()
-    assert all(torch.isfinite(p).all() for p in params)
+    assert opt.state[gain]["step"] == 1 and torch.equal(gain.detach(), before)
 
 
 def test_tensor_hyper_parameters_and_side_streams_change_nothing(M):

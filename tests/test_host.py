@@ -428,3 +428,15 @@ def test_update_products_take_large_tiles_only_where_they_fill_the_gpu():
     assert c.update_class == 0
     (c,) = plan.plan_chunks([(4096, 4096)] * 2, 5, True, 16 << 30)
     assert c.tile_class == 1 and c.update_class == 1
+
+
+def test_rows_only_aol_is_refused_below_its_stated_size():
+    """plan_chunks refuses the rows-only AOL rescaling for a matrix with a side below
+    AOL_ROWS_MIN_SIDE (the map does not contract there), and only that variant."""
+    from muon_amd import plan
+    for shape in [(18, 63), (63, 18), (31, 4096)]:
+        with pytest.raises(ValueError, match="rows-only"):
+            plan.plan_chunks([(256, 256), shape], 4, False, 1 << 30, "aol4_rows")
+        assert plan.plan_chunks([(256, 256), shape], 4, False, 1 << 30, "aol4")
+        assert plan.plan_chunks([(256, 256), shape], 5, True, 1 << 30, "ns5")
+    assert plan.plan_chunks([(plan.AOL_ROWS_MIN_SIDE, 63)], 4, False, 1 << 30, "aol4_rows")
