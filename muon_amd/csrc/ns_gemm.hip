@@ -84,6 +84,28 @@ struct WaitHalves<DPH, 0> {
     static __device__ __forceinline__ void run(int) { NS_WAIT_VMCNT(0); }
 };
 
+// Fragment reads of the main loop: N ds_read_b128 from LDS byte address addr + i * 32 rows, issued
+// through inline assembly so that the waits for them can be placed by hand (wait_frags).
+template <int N, int I = 0>
+struct FragLoad {
+    static __device__ __forceinline__ void run(u32x4 (&f)[N], uint32_t addr) {
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[I]) : "v"(addr), "n"(I * 32 * ROW_BYTES));
+        if constexpr (I + 1 < N) FragLoad<N, I + 1>::run(f, addr);
+    }
+};
+// s_waitcnt lgkmcnt(CNT), tied to the fragment registers the following MFMAs read: the compiler
+// sees them redefined here and cannot move a use above the wait.
+template <int CNT, int TM, int TN>
+__device__ __forceinline__ void wait_frags(u32x4 (&a)[TM], u32x4 (&b)[TN]) {
+    static_assert(CNT >= 0 && CNT < 16, "lgkmcnt is a 4-bit counter");
+    if constexpr (TM == 4 && TN == 2)
+        asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]) : "n"(CNT));
+    else if constexpr (TM == 2 && TN == 2)
+        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : "n"(CNT));
+    else
+        static_assert(TM == 2 && TN == 2, "wait_frags: add the operand list of this wave tile");
+}
+
 // ---------------------------------------------------------------------------------------------
 // Epilogue helpers
 // ---------------------------------------------------------------------------------------------
@@ -487,6 +509,9 @@ template <int BT_, int WGM_, int WGN_, int MINB_, int NHALF_, bool SPLIT_K_>
 struct GemmCfg {
     static constexpr bool SPLIT_K = SPLIT_K_;     // jobs may share a tile's reduction
     static constexpr bool STREAM_STORES = BT_ >= 256;   // see gstore16
+    // A second copy of the k-block without the tests of the first and last blocks (see NS_KBLOCK).
+    // The 256 x 256 class has no registers to spare for the moves between two copies of its loop.
+    static constexpr bool STEADY_LOOP = BT_ < 256;
     static constexpr int BM = BT_, BN = BT_, WGM = WGM_, WGN = WGN_, MINB = MINB_, NHALF = NHALF_;
     static constexpr int NW = WGM * WGN, NT = NW * 64;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
@@ -580,6 +605,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     constexpr int KSTEPS = BK / 16;
     constexpr int DPK = 2 * DPH / KSTEPS;                    // DMA instructions per k-step
     static_assert(2 * DPH % KSTEPS == 0 && DPH % DPK == 0, "DMA instructions must spread evenly");
+    static_assert(KSTEPS % 2 == 0, "the fragments read at a block's last k-step land in buffer 0");
     static_assert(DPK <= TM, "one DMA instruction per row of MFMAs");
 
     const bool round_terms = (flags & MUON_AMD_ROUND_REFERENCE) != 0;
@@ -607,9 +633,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         // ---- fragment addressing (bytes): lane l reads row l%32, chunk 2*ks + l/32 -------------
         const int swz = (lane >> 1) & 7;
         const int c0 = (lane >> 5) ^ swz;
-        const char* const ldsb = reinterpret_cast<const char*>(lds);
-        const char* const pfrag = ldsb + (wm * WM + (lane & 31)) * ROW_BYTES;
-        const char* const qfrag = ldsb + (wn * WN + (lane & 31)) * ROW_BYTES;
+        const uint32_t pfrag_off = (wm * WM + (lane & 31)) * ROW_BYTES;
+        const uint32_t qfrag_off = (wn * WN + (lane & 31)) * ROW_BYTES;
         const int koff[4] = {c0 * 16, (c0 ^ 2) * 16, (c0 ^ 4) * 16, (c0 ^ 6) * 16};
         // the sources of the halves beyond the first ones (set again: the copies made when the
         // first halves were issued are not kept across the epilogue before)
@@ -630,16 +655,24 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
 
         // Fragments are double buffered over k-steps ACROSS blocks: the ds_reads of the next k-step
         // (the first one of block kb+1 included) are issued ahead of the MFMAs of the current one, so
-        // the matrix pipe never waits for LDS latency, not even right after the barrier.
-        bf16x8 af[2][TM], bfr[2][TN];
-#define NS_LOAD_FRAGS(buf_, pf_, qf_, ks_)                                                      \
+        // the matrix pipe never waits for LDS latency, not even right after the barrier.  The reads
+        // and the waits for them are written out (FragLoad, wait_frags): LDS reads return in order,
+        // so "at most TM + TN outstanding" means the fragments of the current k-step have arrived
+        // while those just requested are still in flight.  Left to the compiler, the wait at the
+        // join after the last block's branch covered the reads issued right after the barrier.
+        // The compiler takes a register written by FragLoad as valid at once: between a read and
+        // its wait there must be no place where it may copy that register (no loop edge, no join
+        // of paths that define it differently).
+        u32x4 af[2][TM], bfr[2][TN];
+        const uint32_t pfrag_a = lds_base + pfrag_off;
+        const uint32_t qfrag_a = lds_base + qfrag_off;
+#define NS_LOAD_FRAGS(buf_, sp_, sq_, ks_)                                                      \
     do {                                                                                       \
-        _Pragma("unroll") for (int a_ = 0; a_ < TM; ++a_)                                      \
-            af[buf_][a_] = *reinterpret_cast<const bf16x8*>((pf_) + a_ * 32 * ROW_BYTES + koff[ks_]); \
-        _Pragma("unroll") for (int b_ = 0; b_ < TN; ++b_)                                      \
-            bfr[buf_][b_] = *reinterpret_cast<const bf16x8*>((qf_) + b_ * 32 * ROW_BYTES + koff[ks_]); \
+        FragLoad<TM>::run(af[buf_], pfrag_a + (sp_) * HALF_BYTES + koff[ks_]);                 \
+        FragLoad<TN>::run(bfr[buf_], qfrag_a + (sq_) * HALF_BYTES + koff[ks_]);                \
     } while (0)
-        NS_LOAD_FRAGS(0, pfrag, qfrag + HALF_BYTES, 0);
+        NS_LOAD_FRAGS(0, 0, 1, 0);
+        wait_frags<0>(af[0], bfr[0]);      // (once per tile) nothing in flight on entry to the loop either
 
         // The pair of halves being issued: created at the barrier of block kb (last k-step), its
         // 2*DPH DMA instructions are spread over that k-step and the first KSTEPS-1 of block kb+1,
@@ -651,56 +684,89 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         size_t dk[2] = {0, 0};
         bool dgo[2] = {false, false};
 
+        // One k-block.  STEADY_: a block in the middle of a long reduction -- both halves of the pair
+        // created at the previous barrier and the first half of the pair created at this one exist
+        // (1 <= kb <= nk - 3), so every DMA instruction is issued without a test and the wait before
+        // the barrier is a constant; the first block and the last two take the general form.
+#define NS_KBLOCK(STEADY_)                                                                      \
+    do {                                                                                       \
+        int spn = sp + 2; spn = spn >= NHALF ? spn - NHALF : spn;                              \
+        int sqn = sq + 2; sqn = sqn >= NHALF ? sqn - NHALF : sqn;                              \
+        _Pragma("unroll") for (int ks = 0; ks < KSTEPS; ++ks) {                                \
+            const int cur = ks & 1, nxt = cur ^ 1;                                             \
+            if (ks + 1 < KSTEPS) {                                                             \
+                NS_LOAD_FRAGS(nxt, sp, sq, ks + 1);                                            \
+                wait_frags<TM + TN>(af[cur], bfr[cur]);                                        \
+            } else {                                                                           \
+                /* Every fragment of block kb is in registers.  Block kb+1 has landed once only   \
+                   the younger halves are pending; after the barrier it is visible to all waves   \
+                   and the two slots of block kb are free for the next pair of halves,            \
+                   2kb+NHALF and 2kb+NHALF+1. */                                                  \
+                wait_frags<0>(af[cur], bfr[cur]);                                              \
+                if (STEADY_ || kb + 1 < nk) {                                                  \
+                    if (STEADY_) {                                                             \
+                        NS_WAIT_VMCNT((NHALF - 4) * DPH);                                      \
+                    } else {                                                                   \
+                        const int issued = 2 * nk < 2 * kb + NHALF ? 2 * nk : 2 * kb + NHALF;  \
+                        WaitHalves<DPH, NHALF - 2>::run(issued - (2 * kb + 4));                \
+                    }                                                                          \
+                    __builtin_amdgcn_s_barrier();                                              \
+                    const int h0 = 2 * kb + NHALF;                                             \
+                    ddst[0] = dst0 + sp * HALF_BYTES;            /* h0 % NHALF == 2kb % NHALF */  \
+                    ddst[1] = dst0 + sq * HALF_BYTES;                                          \
+                    dk[0] = static_cast<size_t>(h0 >> 1) * BK;                                 \
+                    dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;                           \
+                    dgo[0] = h0 < 2 * nk;                                                      \
+                    dgo[1] = h0 + 1 < 2 * nk;                                                  \
+                } else {                                                                       \
+                    dgo[0] = dgo[1] = false;     /* last block: nothing left to fetch */       \
+                }                                                                              \
+                /* The first fragments of block kb+1, read under the last MFMAs of block kb.      \
+                   After the last block the same reads go out and their result is not used: the   \
+                   fragment registers then have one definition on every path, so the compiler has \
+                   no reason to copy them while the reads are in flight. */                       \
+                NS_LOAD_FRAGS(nxt, spn, sqn, 0);                                               \
+            }                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);   /* keep these reads ahead of the MFMAs below */  \
+            _Pragma("unroll") for (int a = 0; a < TM; ++a) {                                   \
+                _Pragma("unroll") for (int b = 0; b < TN; ++b)                                 \
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                       \
+                        __builtin_bit_cast(bf16x8, af[cur][a]), __builtin_bit_cast(bf16x8, bfr[cur][b]), acc[a][b], 0, 0, 0); \
+                if (a < DPK) {                                                                 \
+                    /* instruction jj of the current pair: the last k-step starts a pair */    \
+                    const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;                 \
+                    const int h = jj / DPH, j = jj % DPH;                                      \
+                    __builtin_amdgcn_sched_barrier(0);                                         \
+                    if (STEADY_ || dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024); \
+                    __builtin_amdgcn_sched_barrier(0);                                         \
+                }                                                                              \
+            }                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                 \
+        }                                                                                      \
+        /* Nothing is in flight across the end of a k-block: the reads issued before the last     \
+           row of MFMAs have long arrived, and waiting for them here keeps every pending          \
+           fragment inside one copy of this code (a register the compiler moved at a loop edge    \
+           or between the two copies would be moved before its data is there). */                 \
+        wait_frags<0>(af[0], bfr[0]);                                                          \
+        sp = spn;                                                                              \
+        sq = sqn;                                                                              \
+    } while (0)
+
         int sp = 0, sq = 1;                 // ring slots of the P and Q halves of block kb
-        for (int kb = 0; kb < nk; ++kb) {
-            const char* const pf = pfrag + sp * HALF_BYTES;
-            const char* const qf = qfrag + sq * HALF_BYTES;
-            int spn = sp + 2; spn = spn >= NHALF ? spn - NHALF : spn;
-            int sqn = sq + 2; sqn = sqn >= NHALF ? sqn - NHALF : sqn;
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                const int cur = ks & 1, nxt = cur ^ 1;
-                if (ks + 1 < KSTEPS) {
-                    NS_LOAD_FRAGS(nxt, pf, qf, ks + 1);
-                } else if (kb + 1 < nk) {
-                    // Every fragment of block kb is in registers (the barrier waits for this wave's
-                    // LDS reads).  Block kb+1 has landed once only the younger halves are pending;
-                    // after the barrier it is visible to all waves and the two slots of block kb are
-                    // free for the next pair of halves, 2kb+NHALF and 2kb+NHALF+1.
-                    const int issued = 2 * nk < 2 * kb + NHALF ? 2 * nk : 2 * kb + NHALF;
-                    WaitHalves<DPH, NHALF - 2>::run(issued - (2 * kb + 4));
-                    __syncthreads();
-                    const int h0 = 2 * kb + NHALF;
-                    ddst[0] = dst0 + sp * HALF_BYTES;                // h0 % NHALF == 2kb % NHALF
-                    ddst[1] = dst0 + sq * HALF_BYTES;
-                    dk[0] = static_cast<size_t>(h0 >> 1) * BK;
-                    dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;
-                    dgo[0] = h0 < 2 * nk;
-                    dgo[1] = h0 + 1 < 2 * nk;
-                    NS_LOAD_FRAGS(nxt, pfrag + spn * HALF_BYTES, qfrag + sqn * HALF_BYTES, 0);
-                } else {
-                    dgo[0] = dgo[1] = false;     // last block: nothing left to fetch
+        for (int kb = 0; kb < nk;) {
+            if constexpr (Cfg::STEADY_LOOP) {
+                if (kb >= 1 && kb <= nk - 3) {
+                    do {
+                        NS_KBLOCK(true);
+                        ++kb;
+                    } while (kb <= nk - 3);
+                    continue;
                 }
-                __builtin_amdgcn_sched_barrier(0);   // keep these reads ahead of the MFMAs below
-#pragma unroll
-                for (int a = 0; a < TM; ++a) {
-#pragma unroll
-                    for (int b = 0; b < TN; ++b)
-                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][a], bfr[cur][b], acc[a][b], 0, 0, 0);
-                    if (a < DPK) {
-                        // instruction jj of the current pair: the last k-step starts a pair
-                        const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;
-                        const int h = jj / DPH, j = jj % DPH;
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (dgo[h]) dma16(dsrc[h][j] + dk[h], ddst[h] + j * NW * 1024);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
             }
-            sp = spn;
-            sq = sqn;
+            NS_KBLOCK(false);
+            ++kb;
         }
+#undef NS_KBLOCK
 #undef NS_LOAD_FRAGS
         __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
 
