@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define MUON_AMD_ABI_VERSION 2
+#define MUON_AMD_ABI_VERSION 3
 
 #define MUON_AMD_OK        0
 #define MUON_AMD_EINVAL   (-1)   /* bad argument (null pointer, bad size, misaligned table) */
@@ -42,6 +42,9 @@ extern "C" {
                                        (A = X X^T): also leave, per row of the result, partial sums
                                        of |A_ij| in MuonGemmDesc.rowsum (muon.py:779-781 fused into
                                        the product's epilogue) */
+#define MUON_AMD_GEMM_Q_KMAJOR   8  /* muon_amd_ns_gemm: every descriptor of the launch gives its second
+                                       operand k-major (MuonGemmDesc.q_kmajor = 1); muon_amd_ns_gemm_apply
+                                       always takes it that way */
 
 /* How muon_amd_aol_rescale scales the Gram matrix (mode argument). */
 #define MUON_AMD_AOL_SYMMETRIC   0  /* A <- diag(r) A diag(r): the Gram matrix of the rescaled X   */
@@ -90,7 +93,9 @@ typedef struct MuonMatDesc {
     int32_t   part_end;    /* one past the last                                               */
 } MuonMatDesc;
 
-/* One NT GEMM  acc[i][j] = sum_k P[i][k] * Q[j][k]  over a padded matrix, with the epilogue
+/* One GEMM  acc[i][j] = sum_k P[i][k] * Q[j][k]  ("NT": both operands row-major along k; with
+ * q_kmajor = 1 the second operand is given as Q[k][j], leading dimension ldq >= colsn, so that
+ * a X + B X reads X itself and no transposed copy of X is kept) over a padded matrix, with the epilogue
  *     t1 = alpha*acc ; t2 = beta*D[i][j] ; (both rounded to bf16 under ROUND_REFERENCE)
  *     o  = bf16(t1 + t2)          -> C[i][j]  and  CT[j][i]
  *     o2 = bf16(gamma * o)        -> C2[i][j] and  C2T[j][i]
@@ -111,7 +116,7 @@ typedef struct MuonGemmDesc {
      * launch, some with zero; adding a row's entries in slot order gives sum_j |o_ij|).       */
     float*  rowsum;
     int32_t ld_rowsum;                  /* >= colsn / 64                                       */
-    int32_t reserved;                   /* 0                                                   */
+    int32_t q_kmajor;                   /* 0: Q is colsn x K, rows along k; 1: Q is K x colsn   */
 } MuonGemmDesc;
 
 /* One output tile of one matrix, or one share of its reduction.  A tile whose K is long and

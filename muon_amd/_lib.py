@@ -14,11 +14,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MUON_AMD_LIBRARY: path of another build of the library (for comparing builds side by side)
 LIB_PATH = os.environ.get("MUON_AMD_LIBRARY") or os.path.join(_HERE, "libmuon_amd.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 ROUND_REFERENCE = 1
 ROUND_FUSED = 0
 NORM_UNIT = 2
 GEMM_ROWSUM = 4
+GEMM_Q_KMAJOR = 8
 AOL_SYMMETRIC = 0
 AOL_ROWS_ONLY = 1
 SRC_F32 = 0
@@ -36,7 +37,7 @@ GEMM_DESC = np.dtype(
     [("P", "<u8"), ("Q", "<u8"), ("D", "<u8"), ("C", "<u8"), ("CT", "<u8"), ("C2", "<u8"),
      ("C2T", "<u8"), ("ldp", "<i4"), ("ldq", "<i4"), ("ldd", "<i4"), ("ldc", "<i4"),
      ("ldct", "<i4"), ("K", "<i4"), ("rows", "<i4"), ("colsn", "<i4"),
-     ("rowsum", "<u8"), ("ld_rowsum", "<i4"), ("reserved", "<i4")],
+     ("rowsum", "<u8"), ("ld_rowsum", "<i4"), ("q_kmajor", "<i4")],
     align=True)
 TILE_JOB = np.dtype([("desc", "<i4"), ("i0", "<i4"), ("j0", "<i4"), ("diag", "<i4"), ("k0", "<i4"),
                      ("k1", "<i4"), ("part_base", "<i4"), ("split", "<i4")], align=True)

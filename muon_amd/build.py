@@ -42,7 +42,7 @@ def _vregs(text: str) -> frozenset:
 
 def check_fragment_waits(asm_text: str) -> int:
     """Walks the control-flow graph of every ns_gemm_kernel in a hipcc -S listing.  A register that an
-    inline-assembly ds_read_b128 has requested is pending until a `s_waitcnt lgkmcnt(n)` leaves at
+    inline-assembly LDS read (ds_read_b128, ds_read_b64_tr_b16) has requested is pending until a `s_waitcnt lgkmcnt(n)` leaves at
     most n younger requests outstanding (LDS reads return in order).  Raises if any instruction --
     a copy the register allocator put at a loop edge, an address computation, an MFMA -- names a
     pending register: it would see the register before its data.  Returns the number of such reads
@@ -78,7 +78,7 @@ def check_fragment_waits(asm_text: str) -> int:
                     if m:
                         n = int(m.group(1))
                         pend = pend[len(pend) - n:] if n else ()
-                elif op == "ds_read_b128" and from_asm:
+                elif op in ("ds_read_b128", "ds_read_b64_tr_b16") and from_asm:
                     dst, addr = t.split(None, 1)[1].split(",")[:2]
                     if any(p & _vregs(addr) for p in pend):
                         raise RuntimeError(f"ns_gemm.hip: line {line_no} of the listing reads LDS through a pending register: {t}")

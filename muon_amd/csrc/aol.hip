@@ -126,7 +126,7 @@ int muon_amd_validate_aol(const MuonAolDesc* descs, int nmat, const int32_t* row
     MUON_REQUIRE(row_prefix[0] == 0 && seg_prefix[0] == 0, "validate_aol: prefix must start at 0");
     for (int i = 0; i < nmat; ++i) {
         const MuonAolDesc& d = descs[i];
-        MUON_REQUIRE(d.xr && d.xc && d.gram && d.rvec, "aol desc %d: null pointer", i);
+        MUON_REQUIRE(d.xr && d.gram && d.rvec, "aol desc %d: null pointer", i);
         MUON_REQUIRE(d.m_p > 0 && d.n_p > 0 && d.m_p % 8 == 0 && d.n_p % 8 == 0 &&
                          d.m_p % AOL_ROWS_PER_BLOCK == 0 && d.n_p % AOL_ROWS_PER_BLOCK == 0,
                      "aol desc %d: padded sizes %d x %d", i, d.m_p, d.n_p);
@@ -140,7 +140,8 @@ int muon_amd_validate_aol(const MuonAolDesc* descs, int nmat, const int32_t* row
         MUON_REQUIRE(row_prefix[i + 1] - row_prefix[i] == d.m_p / AOL_ROWS_PER_BLOCK,
                      "aol desc %d: row prefix gives %d blocks, need %d", i, row_prefix[i + 1] - row_prefix[i],
                      d.m_p / AOL_ROWS_PER_BLOCK);
-        const int need[3] = {d.m_p / AOL_ROWS_PER_BLOCK, d.n_p / AOL_ROWS_PER_BLOCK, d.m_p / AOL_ROWS_PER_BLOCK};
+        // (no blocks for the rows of a transposed copy that is not kept)
+        const int need[3] = {d.m_p / AOL_ROWS_PER_BLOCK, d.xc ? d.n_p / AOL_ROWS_PER_BLOCK : 0, d.m_p / AOL_ROWS_PER_BLOCK};
         for (int k = 0; k < 3; ++k)
             MUON_REQUIRE(seg_prefix[3 * i + k + 1] - seg_prefix[3 * i + k] == need[k],
                          "aol desc %d: segment %d has %d blocks, need %d", i, k,

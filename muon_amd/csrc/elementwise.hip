@@ -235,7 +235,9 @@ __global__ __launch_bounds__(64) void norm_finalize_kernel(const MuonMatDesc* __
 }
 
 // ------------------------------------------------------------------------------------------
-// normalise + transpose + zero pad:  direct = bf16(u / denom), transp = direct^T
+// normalise (+ transpose) + zero pad:  direct = bf16(u / denom) and / or transp = its transpose;
+// an orientation whose pointer is null is not written (the iteration keeps one orientation only:
+// the parameter's own for a wide matrix, the transposed one for a tall matrix)
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4e __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x4e gld4u(const uint16_t* p) {
@@ -293,11 +295,12 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
         u32x4e o;
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = v[2 * k] | (static_cast<uint32_t>(v[2 * k + 1]) << 16);
-        gst4u(d.direct + static_cast<int64_t>(gr) * d.ld_direct + gc, o);
+        if (d.direct) gst4u(d.direct + static_cast<int64_t>(gr) * d.ld_direct + gc, o);
         uint2* const dst = reinterpret_cast<uint2*>(&tile[r][cc / 2]);
         dst[0] = make_uint2(o[0], o[1]);
         dst[1] = make_uint2(o[2], o[3]);
     }
+    if (!d.transp) return;                 // (the same for every thread of the block)
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < (NT_TILE / 2) * CH / 256; ++i) {
@@ -537,8 +540,10 @@ int muon_amd_validate_mats(const MuonMatDesc* descs, int nmat, const int32_t* bl
                          d.ld_transp % 8 == 0,
                      "mat %d: leading dimensions %d/%d for padded %dx%d", i, d.ld_direct, d.ld_transp,
                      d.rows_p, d.cols_p);
-        MUON_REQUIRE(d.grad && d.u && d.direct && d.transp && d.result && d.partials && d.denom,
+        MUON_REQUIRE(d.grad && d.u && (d.direct || d.transp) && d.partials && d.denom,
                      "mat %d: null workspace or source pointer", i);
+        MUON_REQUIRE(!d.result || d.result == d.direct,
+                     "mat %d: the result of a run without iterations is the normalised matrix in the parameter's orientation", i);
         MUON_REQUIRE(d.param || d.out, "mat %d: neither param nor out given", i);
         MUON_REQUIRE(d.src_dtype == MUON_AMD_SRC_F32 || d.src_dtype == MUON_AMD_SRC_BF16,
                      "mat %d: src_dtype=%d", i, d.src_dtype);

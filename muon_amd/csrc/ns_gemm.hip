@@ -93,6 +93,23 @@ struct FragLoad {
         if constexpr (I + 1 < N) FragLoad<N, I + 1>::run(f, addr);
     }
 };
+// The same for an operand that lies k-major in LDS (row = k, the tile's columns along the row: X
+// itself as the second operand of B X): ds_read_b64_tr_b16 takes, in every group of 16 lanes, from
+// lane 4r + c the address of columns 4c .. 4c+3 of row r of a 4 x 16 block and hands lane j the four
+// rows of column j.  With lanes 0..15 / 16..31 on columns 0..15 / 16..31 of rows 0..3 and lanes 32..63
+// on rows 8..11, two such reads (rows +0 and +4) leave lane l with k = 8 (l / 32) .. + 7 of column
+// l % 32: exactly the second operand of v_mfma_f32_32x32x16_bf16 (checked on the device).
+// f[2 i], f[2 i + 1]: the two halves of fragment i; addr[i]: its per-lane LDS byte address (the
+// 64-byte column blocks of a row are XOR-swizzled with row & 3, so it depends on i).
+template <int N, int ROWQ, int I = 0>
+struct FragLoadTr {
+    static __device__ __forceinline__ void run(u32x2 (&f)[2 * N], const uint32_t (&addr)[N], uint32_t base) {
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:0" : "=v"(f[2 * I]) : "v"(addr[I] + base));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(f[2 * I + 1]) : "v"(addr[I] + base), "n"(4 * ROWQ));
+        if constexpr (I + 1 < N) FragLoadTr<N, ROWQ, I + 1>::run(f, addr, base);
+    }
+};
+
 // s_waitcnt lgkmcnt(CNT), tied to the fragment registers the following MFMAs read: the compiler
 // sees them redefined here and cannot move a use above the wait.
 template <int CNT, int TM, int TN>
@@ -104,6 +121,17 @@ __device__ __forceinline__ void wait_frags(u32x4 (&a)[TM], u32x4 (&b)[TN]) {
         asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]) : "n"(CNT));
     else
         static_assert(TM == 2 && TN == 2, "wait_frags: add the operand list of this wave tile");
+}
+template <int CNT, int TM, int TN2>
+__device__ __forceinline__ void wait_frags_tr(u32x4 (&a)[TM], u32x2 (&b)[TN2]) {
+    static_assert(CNT >= 0 && CNT < 16, "lgkmcnt is a 4-bit counter");
+    if constexpr (TM == 4 && TN2 == 4)
+        asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]),
+                     "+v"(b[2]), "+v"(b[3]) : "n"(CNT));
+    else if constexpr (TM == 2 && TN2 == 4)
+        asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a[0]), "+v"(a[1]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]) : "n"(CNT));
+    else
+        static_assert(TM == 2 && TN2 == 4, "wait_frags_tr: add the operand list of this wave tile");
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -546,7 +574,10 @@ struct GemmCfg {
 // APPLY: the launch is the last update product of the iteration and its epilogue takes the
 // parameter step (mats[job.desc] describes the parameter of the job's matrix; `sc`, when given,
 // holds {lr, wd_factor} in device memory and overrides the by-value arguments).
-template <typename Cfg, bool APPLY>
+// QK: the second operand is given k-major, Q[k][j] with leading dimension ldq (acc[i][j] = sum_k
+// P[i][k] Q[k][j]: the update a X + B X reads X itself, no transposed copy of it exists); its
+// half-stage is then BK rows of BN columns, fetched in the same 1 KiB pieces.
+template <typename Cfg, bool APPLY, bool QK>
 __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     const MuonGemmDesc* __restrict__ descs, const MuonTileJob* __restrict__ jobs, int njobs, float alpha,
     float beta, float gamma, int flags, float* __restrict__ split_partials,
@@ -555,6 +586,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     constexpr int NW = Cfg::NW, WGN = Cfg::WGN, WM = Cfg::WM, WN = Cfg::WN;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, HALF_BYTES = Cfg::HALF_BYTES, DPH = Cfg::DPH;
     constexpr int NHALF = Cfg::NHALF, NPRE = Cfg::NPRE;
+    constexpr int ROWQ = Cfg::BN * 2;           // bytes of one k-row of a k-major Q half-stage
+    static_assert(!APPLY || QK, "the parameter step rides the update product, whose second operand is k-major");
     extern __shared__ __align__(16) uint16_t lds[];
     const int tid = threadIdx.x;
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
@@ -573,22 +606,34 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     const int wm = wave / WGN, wn = wave % WGN;                                                \
     const int gchunk = (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));                         \
     const uint32_t dst0 = lds_base + wave * 1024
+    // k-major Q: piece (j*NW + wave) of the half-stage is 1024 / ROWQ whole k-rows; lane -> k-row
+    // and 16-byte position in it; the 64-byte block at position pb of row k holds the row's block
+    // pb ^ (k & 3) (the transposing fragment reads of four consecutive k then hit different banks).
     const uint16_t* srcp[DPH];
     const uint16_t* srcq[DPH];
+    size_t qstep;                               // elements from one k-block of Q to the next
 #define NS_SET_SOURCES(job_, d_)                                                               \
     do {                                                                                       \
         _Pragma("unroll") for (int j_ = 0; j_ < DPH; ++j_) {                                   \
             const int r_ = (j_ * NW + wave) * 8 + (lane >> 3);                                 \
             srcp[j_] = (d_).P + static_cast<size_t>((job_).i0 + r_) * (d_).ldp + (job_).k0 + gchunk * 8; \
-            srcq[j_] = (d_).Q + static_cast<size_t>((job_).j0 + r_) * (d_).ldq + (job_).k0 + gchunk * 8; \
+            if constexpr (QK) {                                                                \
+                const int o_ = (j_ * NW + wave) * 1024 + lane * 16;                            \
+                const int k_ = o_ / ROWQ, w_ = o_ % ROWQ;                                      \
+                const int col_ = (((w_ >> 6) ^ (k_ & 3)) << 5) + ((w_ & 63) >> 1);             \
+                srcq[j_] = (d_).Q + static_cast<size_t>((job_).k0 + k_) * (d_).ldq + (job_).j0 + col_; \
+            } else {                                                                           \
+                srcq[j_] = (d_).Q + static_cast<size_t>((job_).j0 + r_) * (d_).ldq + (job_).k0 + gchunk * 8; \
+            }                                                                                  \
         }                                                                                      \
+        qstep = QK ? static_cast<size_t>(BK) * (d_).ldq : static_cast<size_t>(BK);             \
     } while (0)
 
     // half h = 2*kb (+1): P (Q) rows of k-block kb, into ring slot h % NHALF
-#define NS_ISSUE_HALF(src_, kb_, slot_)                                                        \
+#define NS_ISSUE_HALF(src_, step_, kb_, slot_)                                                 \
     do {                                                                                       \
         _Pragma("unroll") for (int j_ = 0; j_ < DPH; ++j_)                                     \
-            dma16(src_[j_] + static_cast<size_t>(kb_) * BK,                                    \
+            dma16(src_[j_] + static_cast<size_t>(kb_) * (step_),                               \
                   dst0 + (slot_) * HALF_BYTES + j_ * NW * 1024);                               \
     } while (0)
     // the first halves of a job, h in [H0_, H1_) and below 2*nk_: P0 Q0 P1 Q1 P2 ... into slots 0 1 2 ...
@@ -596,8 +641,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
     do {                                                                                       \
         _Pragma("unroll") for (int h_ = (H0_); h_ < (H1_); ++h_) {                             \
             if (h_ < 2 * (nk_)) {                                                              \
-                if (h_ & 1) NS_ISSUE_HALF(srcq, h_ >> 1, h_);                                  \
-                else NS_ISSUE_HALF(srcp, h_ >> 1, h_);                                         \
+                if (h_ & 1) NS_ISSUE_HALF(srcq, qstep, h_ >> 1, h_);                           \
+                else NS_ISSUE_HALF(srcp, static_cast<size_t>(BK), h_ >> 1, h_);                \
             }                                                                                  \
         }                                                                                      \
     } while (0)
@@ -635,6 +680,16 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         const int c0 = (lane >> 5) ^ swz;
         const uint32_t pfrag_off = (wm * WM + (lane & 31)) * ROW_BYTES;
         const uint32_t qfrag_off = (wn * WN + (lane & 31)) * ROW_BYTES;
+        // k-major Q: lane l addresses row 8 (l / 32) + (l % 16) / 4 of the k-step, columns
+        // 32 b + 16 ((l / 16) % 2) + 4 (l % 4) .. + 3 of the wave's 64, in the swizzled block
+        uint32_t qtr_off[TN];
+        if constexpr (QK) {
+            const int r4 = (lane & 15) >> 2;
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+                qtr_off[b] = ((lane >> 5) * 8 + r4) * ROWQ + (((wn * (WN / 32) + b) ^ r4) << 6) +
+                             ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
+        }
         const int koff[4] = {c0 * 16, (c0 ^ 2) * 16, (c0 ^ 4) * 16, (c0 ^ 6) * 16};
         // the sources of the halves beyond the first ones (set again: the copies made when the
         // first halves were issued are not kept across the epilogue before)
@@ -664,15 +719,25 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         // its wait there must be no place where it may copy that register (no loop edge, no join
         // of paths that define it differently).
         u32x4 af[2][TM], bfr[2][TN];
+        u32x2 btr[2][2 * TN];               // k-major Q: the halves (k 0..3, k 4..7 of a lane) of its fragments
+        constexpr int NFRAG = TM + (QK ? 2 * TN : TN);      // LDS reads of one k-step
         const uint32_t pfrag_a = lds_base + pfrag_off;
         const uint32_t qfrag_a = lds_base + qfrag_off;
 #define NS_LOAD_FRAGS(buf_, sp_, sq_, ks_)                                                      \
     do {                                                                                       \
         FragLoad<TM>::run(af[buf_], pfrag_a + (sp_) * HALF_BYTES + koff[ks_]);                 \
-        FragLoad<TN>::run(bfr[buf_], qfrag_a + (sq_) * HALF_BYTES + koff[ks_]);                \
+        if constexpr (QK)                                                                      \
+            FragLoadTr<TN, ROWQ>::run(btr[buf_], qtr_off, lds_base + (sq_) * HALF_BYTES + (ks_) * 16 * ROWQ); \
+        else                                                                                   \
+            FragLoad<TN>::run(bfr[buf_], qfrag_a + (sq_) * HALF_BYTES + koff[ks_]);            \
+    } while (0)
+#define NS_WAIT_FRAGS(CNT_, buf_)                                                               \
+    do {                                                                                       \
+        if constexpr (QK) wait_frags_tr<CNT_>(af[buf_], btr[buf_]);                            \
+        else wait_frags<CNT_>(af[buf_], bfr[buf_]);                                            \
     } while (0)
         NS_LOAD_FRAGS(0, 0, 1, 0);
-        wait_frags<0>(af[0], bfr[0]);      // (once per tile) nothing in flight on entry to the loop either
+        NS_WAIT_FRAGS(0, 0);               // (once per tile) nothing in flight on entry to the loop either
 
         // The pair of halves being issued: created at the barrier of block kb (last k-step), its
         // 2*DPH DMA instructions are spread over that k-step and the first KSTEPS-1 of block kb+1,
@@ -682,6 +747,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
         const uint16_t* const* dsrc[2] = {(NHALF & 1) ? srcq : srcp, (NHALF & 1) ? srcp : srcq};
         uint32_t ddst[2] = {0, 0};
         size_t dk[2] = {0, 0};
+        const size_t dstep[2] = {(NHALF & 1) ? qstep : static_cast<size_t>(BK), (NHALF & 1) ? static_cast<size_t>(BK) : qstep};
         bool dgo[2] = {false, false};
 
         // One k-block.  STEADY_: a block in the middle of a long reduction -- both halves of the pair
@@ -696,13 +762,13 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             const int cur = ks & 1, nxt = cur ^ 1;                                             \
             if (ks + 1 < KSTEPS) {                                                             \
                 NS_LOAD_FRAGS(nxt, sp, sq, ks + 1);                                            \
-                wait_frags<TM + TN>(af[cur], bfr[cur]);                                        \
+                NS_WAIT_FRAGS(NFRAG, cur);                                                     \
             } else {                                                                           \
                 /* Every fragment of block kb is in registers.  Block kb+1 has landed once only   \
                    the younger halves are pending; after the barrier it is visible to all waves   \
                    and the two slots of block kb are free for the next pair of halves,            \
                    2kb+NHALF and 2kb+NHALF+1. */                                                  \
-                wait_frags<0>(af[cur], bfr[cur]);                                              \
+                NS_WAIT_FRAGS(0, cur);                                                         \
                 if (STEADY_ || kb + 1 < nk) {                                                  \
                     if (STEADY_) {                                                             \
                         NS_WAIT_VMCNT((NHALF - 4) * DPH);                                      \
@@ -714,8 +780,8 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
                     const int h0 = 2 * kb + NHALF;                                             \
                     ddst[0] = dst0 + sp * HALF_BYTES;            /* h0 % NHALF == 2kb % NHALF */  \
                     ddst[1] = dst0 + sq * HALF_BYTES;                                          \
-                    dk[0] = static_cast<size_t>(h0 >> 1) * BK;                                 \
-                    dk[1] = static_cast<size_t>((h0 + 1) >> 1) * BK;                           \
+                    dk[0] = static_cast<size_t>(h0 >> 1) * dstep[0];                           \
+                    dk[1] = static_cast<size_t>((h0 + 1) >> 1) * dstep[1];                     \
                     dgo[0] = h0 < 2 * nk;                                                      \
                     dgo[1] = h0 + 1 < 2 * nk;                                                  \
                 } else {                                                                       \
@@ -729,9 +795,13 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             }                                                                                  \
             __builtin_amdgcn_sched_barrier(0);   /* keep these reads ahead of the MFMAs below */  \
             _Pragma("unroll") for (int a = 0; a < TM; ++a) {                                   \
-                _Pragma("unroll") for (int b = 0; b < TN; ++b)                                 \
+                _Pragma("unroll") for (int b = 0; b < TN; ++b) {                               \
+                    u32x4 qv;                                                                  \
+                    if constexpr (QK) qv = u32x4{btr[cur][2 * b].x, btr[cur][2 * b].y, btr[cur][2 * b + 1].x, btr[cur][2 * b + 1].y}; \
+                    else qv = bfr[cur][b];                                                     \
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(                       \
-                        __builtin_bit_cast(bf16x8, af[cur][a]), __builtin_bit_cast(bf16x8, bfr[cur][b]), acc[a][b], 0, 0, 0); \
+                        __builtin_bit_cast(bf16x8, af[cur][a]), __builtin_bit_cast(bf16x8, qv), acc[a][b], 0, 0, 0); \
+                }                                                                              \
                 if (a < DPK) {                                                                 \
                     /* instruction jj of the current pair: the last k-step starts a pair */    \
                     const int jj = (ks + 1 < KSTEPS ? (ks + 1) * DPK : 0) + a;                 \
@@ -747,7 +817,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
            row of MFMAs have long arrived, and waiting for them here keeps every pending          \
            fragment inside one copy of this code (a register the compiler moved at a loop edge    \
            or between the two copies would be moved before its data is there). */                 \
-        wait_frags<0>(af[0], bfr[0]);                                                          \
+        NS_WAIT_FRAGS(0, 0);                                                                   \
         sp = spn;                                                                              \
         sq = sqn;                                                                              \
     } while (0)
@@ -767,6 +837,7 @@ __global__ __launch_bounds__(Cfg::NT, Cfg::MINB) void ns_gemm_kernel(
             ++kb;
         }
 #undef NS_KBLOCK
+#undef NS_WAIT_FRAGS
 #undef NS_LOAD_FRAGS
         __syncthreads();            // every wave is done reading the ring: LDS becomes staging space
 
@@ -971,9 +1042,9 @@ struct DeviceState {
 static DeviceState g_devices[kMaxDevices];
 static std::mutex g_devices_mutex;
 
-template <typename Cfg, bool APPLY>
+template <typename Cfg, bool APPLY, bool QK>
 static int raise_lds_limit() {
-    auto kern = ns_gemm_kernel<Cfg, APPLY>;
+    auto kern = ns_gemm_kernel<Cfg, APPLY, QK>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                             static_cast<int>(Cfg::LDS_BYTES)) != hipSuccess) {
         (void)hipGetLastError();
@@ -1007,10 +1078,12 @@ static int device_setup(const DeviceState** out) {
             set_error("device %d is %s: this library holds gfx950 (MI355X) code only", dev, prop.gcnArchName);
             return MUON_AMD_EDEVICE;
         }
-        int rc = raise_lds_limit<Cfg0, false>();
-        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg0, true>();
-        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, false>();
-        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, true>();
+        int rc = raise_lds_limit<Cfg0, false, false>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg0, false, true>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg0, true, true>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, false, false>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, false, true>();
+        if (rc == MUON_AMD_OK) rc = raise_lds_limit<Cfg1, true, true>();
         if (rc != MUON_AMD_OK) return rc;
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
@@ -1040,11 +1113,15 @@ static int launch_gemm(const DeviceState& st, const MuonGemmDesc* descs, const M
     const int resident = st.num_cus * Cfg::MINB;
     const int grid = njobs < resident ? njobs : resident;
     if (ap.mats)
-        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, true>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, true, true>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+                           njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
+                           ap.wd_factor, ap.scalars);
+    else if (flags & MUON_AMD_GEMM_Q_KMAJOR)
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false, true>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
                            njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
                            ap.wd_factor, ap.scalars);
     else
-        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
+        hipLaunchKernelGGL((ns_gemm_kernel<Cfg, false, false>), dim3(grid), dim3(Cfg::NT), Cfg::LDS_BYTES, s, descs, jobs,
                            njobs, alpha, beta, gamma, flags, split_partials, split_counters, ap.mats, ap.neg_lr,
                            ap.wd_factor, ap.scalars);
     return check_launch("ns_gemm");
@@ -1101,8 +1178,13 @@ int muon_amd_validate_gemm(const MuonGemmDesc* descs, int ndesc, const MuonTileJ
         MUON_REQUIRE(d.K > 0 && d.K % BK == 0, "gemm desc %d: K=%d is not a positive multiple of %d", i, d.K, BK);
         MUON_REQUIRE(d.rows > 0 && d.colsn > 0 && d.rows % TR == 0 && d.colsn % TC == 0,
                      "gemm desc %d: output %dx%d is not in tiles of %dx%d", i, d.rows, d.colsn, TR, TC);
-        MUON_REQUIRE(d.ldp >= d.K && d.ldq >= d.K && d.ldp % 8 == 0 && d.ldq % 8 == 0,
-                     "gemm desc %d: ldp=%d ldq=%d K=%d", i, d.ldp, d.ldq, d.K);
+        MUON_REQUIRE(d.q_kmajor == 0 || d.q_kmajor == 1, "gemm desc %d: q_kmajor=%d", i, d.q_kmajor);
+        MUON_REQUIRE(d.q_kmajor == descs[0].q_kmajor, "gemm desc %d: one launch takes its second operands in one layout", i);
+        MUON_REQUIRE(d.ldp >= d.K && d.ldq >= (d.q_kmajor ? d.colsn : d.K) && d.ldp % 8 == 0 && d.ldq % 8 == 0,
+                     "gemm desc %d: ldp=%d ldq=%d K=%d cols %d (second operand %s)", i, d.ldp, d.ldq, d.K, d.colsn,
+                     d.q_kmajor ? "k-major" : "row-major");
+        MUON_REQUIRE(!d.q_kmajor || !(d.C && (d.C == d.Q || d.C2 == d.Q)),
+                     "gemm desc %d: a k-major second operand is read by every tile of its column block and cannot be overwritten in place", i);
         MUON_REQUIRE(!d.D || (d.ldd >= d.colsn && d.ldd % 8 == 0), "gemm desc %d: ldd=%d cols %d", i, d.ldd, d.colsn);
         MUON_REQUIRE(!(d.C || d.C2) || (d.ldc >= d.colsn && d.ldc % 8 == 0), "gemm desc %d: ldc=%d cols %d", i, d.ldc, d.colsn);
         MUON_REQUIRE(!(d.CT || d.C2T) || (d.ldct >= d.rows && d.ldct % 8 == 0),
@@ -1179,7 +1261,8 @@ int muon_amd_ns_gemm_apply(const MuonGemmDesc* descs_dev, const MuonTileJob* job
     const DeviceState* st = nullptr;
     const int rc = device_setup(&st);
     if (rc != MUON_AMD_OK) return rc;
-    return launch_gemm_class(*st, tile_class, descs_dev, jobs_dev, njobs, alpha, beta, 0.f, flags, nullptr, nullptr,
+    return launch_gemm_class(*st, tile_class, descs_dev, jobs_dev, njobs, alpha, beta, 0.f,
+                             flags | MUON_AMD_GEMM_Q_KMAJOR, nullptr, nullptr,
                              ApplyLaunch{mats_dev, -lr, wd_factor, scalars_dev}, static_cast<hipStream_t>(stream));
 }
 

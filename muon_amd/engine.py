@@ -9,9 +9,6 @@ import torch
 from . import _lib, plan as _plan
 
 DEFAULT_WORKSPACE_CAP = int(os.environ.get("MUON_AMD_WORKSPACE_BYTES", 16 << 30))
-# Measurement knob: 0 runs the parameter step as a launch of its own after the last update product
-# instead of inside that product's epilogue.
-FOLD_APPLY = os.environ.get("MUON_AMD_FOLD_APPLY", "1") != "0"
 
 
 def require_gpu_tensor(t: torch.Tensor, what: str) -> None:
@@ -88,14 +85,14 @@ class _ChunkRuntime:
         for ph in range(_plan.N_PHASES):
             if ph == _plan.PH_POLY_FULL and chunk.poly_full_jobs is None:
                 continue
-            jobs = (chunk.syrk_jobs if ph == _plan.PH_SYRK else
+            jobs = (chunk.syrk_jobs if ph in (_plan.PH_SYRK, _plan.PH_SYRK_ODD) else
                     chunk.sym_jobs if ph == _plan.PH_POLY else
                     chunk.poly_full_jobs if ph == _plan.PH_POLY_FULL else chunk.full_jobs)
             full = ph in (_plan.PH_UPD_EVEN, _plan.PH_UPD_ODD, _plan.PH_UPD_LAST)
             _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(gemm[ph]), chunk.nmat,
                                                   _lib.host_ptr(jobs), len(jobs),
                                                   chunk.update_class if full else chunk.tile_class,
-                                                  chunk.split_slots if ph == _plan.PH_SYRK else 0),
+                                                  chunk.split_slots if ph in (_plan.PH_SYRK, _plan.PH_SYRK_ODD) else 0),
                        "validate_gemm")
         self.mat_template = chunk.mat_descs(base)
         # one static device blob: gemm descs | sym jobs | full jobs | block prefix | tile prefix |
@@ -244,7 +241,7 @@ class _ChunkRuntime:
         norm_flags = flags | (_lib.NORM_UNIT if c.aol else 0)
         _launch("norm_finalize", c.nblocks * 4, lambda: _lib.check(lib.muon_amd_norm_finalize(
             mats, c.nmat, eps, norm_flags, s), "norm_finalize"))
-        _launch("normalize", elts * 2 + padded * 4, lambda: _lib.check(lib.muon_amd_normalize(
+        _launch("normalize", elts * 2 + padded * 2, lambda: _lib.check(lib.muon_amd_normalize(
             mats, self.tile_prefix_ptr, c.nmat, c.ntiles, s), "normalize"))
         flops = {
             _plan.PH_SYRK: sum(lay.m * (lay.m + 1) * lay.n for lay in c.layouts),
@@ -254,7 +251,7 @@ class _ChunkRuntime:
 
         def gemm(name, ph, it, jobs_ptr, njobs, work, extra_flags=0):
             al, be, ga = c.phase_scalars(ph, it)
-            split = ph == _plan.PH_SYRK
+            split = ph in (_plan.PH_SYRK, _plan.PH_SYRK_ODD)
             tile_class = c.update_class if jobs_ptr == self.full_jobs_ptr else c.tile_class
             _launch(name, work, lambda: _lib.check(lib.muon_amd_ns_gemm(
                 self.gemm_ptr[ph], jobs_ptr, njobs, tile_class, al, be, ga, flags | extra_flags,
@@ -263,8 +260,8 @@ class _ChunkRuntime:
 
         for it in range(c.steps):
             first_aol = c.aol and it == 0
-            gemm("ns_gemm/syrk", _plan.PH_SYRK, it, self.syrk_jobs_ptr, len(c.syrk_jobs), flops[_plan.PH_SYRK],
-                 _lib.GEMM_ROWSUM if first_aol else 0)
+            gemm("ns_gemm/syrk", _plan.PH_SYRK if it % 2 == 0 else _plan.PH_SYRK_ODD, it, self.syrk_jobs_ptr,
+                 len(c.syrk_jobs), flops[_plan.PH_SYRK], _lib.GEMM_ROWSUM if first_aol else 0)
             if first_aol:
                 # muon.py:776-785: the row sums of |A| come out of the product's epilogue as partial
                 # sums (one small launch adds them up), then X and A are rescaled in place (A becomes
@@ -275,7 +272,7 @@ class _ChunkRuntime:
                     self.aol_ptr, self.aol_row_prefix_ptr, c.nmat, int(c.aol_row_prefix[-1]), eps, s),
                     "aol_rowsum_finalize"))
                 mode = _lib.AOL_ROWS_ONLY if c.variant == "aol4_rows" else _lib.AOL_SYMMETRIC
-                _launch("aol_rescale", 2 * gram_bytes + 8 * padded, lambda: _lib.check(lib.muon_amd_aol_rescale(
+                _launch("aol_rescale", 2 * gram_bytes + 4 * padded, lambda: _lib.check(lib.muon_amd_aol_rescale(
                     self.aol_ptr, self.aol_seg_prefix_ptr, c.nmat, int(c.aol_seg_prefix[-1]), mode, s),
                     "aol_rescale"))
             if first_aol and c.variant == "aol4_rows":
@@ -284,16 +281,16 @@ class _ChunkRuntime:
                      2 * flops[_plan.PH_POLY])
             else:
                 gemm("ns_gemm/poly", _plan.PH_POLY, it, self.sym_jobs_ptr, len(c.sym_jobs), flops[_plan.PH_POLY])
-            if it == c.steps - 1 and FOLD_APPLY:
+            if it == c.steps - 1:
                 # the last update product takes the parameter step in its epilogue (muon.py:14, 98-99)
                 al, be, _ = c.phase_scalars(_plan.PH_UPD_LAST, it)
                 _launch("ns_gemm/update_apply", f_upd, lambda: _lib.check(lib.muon_amd_ns_gemm_apply(
                     self.gemm_ptr[_plan.PH_UPD_LAST], self.full_jobs_ptr, len(c.full_jobs), c.update_class, al, be,
                     flags, mats, lr, wd_factor, sc_apply, s), "ns_gemm_apply"))
                 return
-            ph = _plan.PH_UPD_LAST if it == c.steps - 1 else (_plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD)
-            gemm("ns_gemm/update", ph, it, self.full_jobs_ptr, len(c.full_jobs), f_upd)
-        # no iteration (steps == 0), or the fused step switched off: a launch of its own
+            gemm("ns_gemm/update", _plan.PH_UPD_EVEN if it % 2 == 0 else _plan.PH_UPD_ODD, it, self.full_jobs_ptr,
+                 len(c.full_jobs), f_upd, _lib.GEMM_Q_KMAJOR)
+        # no iteration (steps == 0): the parameter step is a launch of its own
         _launch("apply", apply_bytes, lambda: _lib.check(lib.muon_amd_apply(
             mats, self.block_prefix_ptr, c.nmat, c.nblocks, lr, wd_factor, sc_apply, s), "apply"))
 

@@ -6,9 +6,12 @@ one apply launch, however many matrices it holds.  Chunks exist only to bound th
 workspace; they share one workspace and run back to back on the stream.
 
 Per matrix (m = min(rows, cols), n = max(rows, cols), padded to the chunk's GEMM tile) the
-workspace holds X (m x n), two copies of X^T (n x m, ping-pong), A, B and c*A (m x m).  The
-un-normalised bf16 update produced by the momentum kernel is parked in the second X^T buffer,
-which the iteration does not touch before the normalise kernel has consumed it.
+workspace holds two m x n buffers X0 and X1 (the iterate and its successor: the update product
+a X + B X reads X itself as its k-major second operand, every tile of a column block reading all
+rows of it, so it cannot be overwritten in place), and A, B, c*A (m x m): 2 m n + 3 m^2 elements
+against the reference's A, B, C beside X (muon.py:765-767).  No transposed copy of X exists.  The
+un-normalised bf16 update produced by the momentum kernel is parked in X1, which the iteration does
+not touch before the normalise kernel has consumed it.
 """
 from __future__ import annotations
 
@@ -49,8 +52,9 @@ RESIDENT_BIG_TILE_WORKGROUPS = 256      # one 256 x 256 workgroup per CU of an M
 LD_PAD = int(os.environ.get("MUON_AMD_LD_PAD", "0"))
 _ALIGN = 256
 
-PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST, PH_POLY_FULL = range(6)
-N_PHASES = 6
+# X X^T and the update of an even iteration read X0 (and the update writes X1), those of an odd one X1
+PH_SYRK, PH_POLY, PH_UPD_EVEN, PH_UPD_ODD, PH_UPD_LAST, PH_POLY_FULL, PH_SYRK_ODD = range(7)
+N_PHASES = 7
 ROWSUM_SLOT = 64                        # columns per slot of the fused row sums (the wave tile's width)
 
 
@@ -98,14 +102,14 @@ class MatLayout:
     mp: int
     np_: int
     wide: bool            # rows <= cols: X is the matrix itself; else X is its transpose
-    off: dict = field(default_factory=dict)   # byte offsets of X, XT0, XT1, A, B, CA
+    off: dict = field(default_factory=dict)   # byte offsets of X0, X1, A, B, CA
 
     @property
     def ldn(self) -> int:     # leading dimension of X (rows of length np_)
         return self.np_ + LD_PAD
 
     @property
-    def ldm(self) -> int:     # leading dimension of X^T, A, B, c*A (rows of length mp)
+    def ldm(self) -> int:     # leading dimension of A, B, c*A (rows of length mp)
         return self.mp + LD_PAD
 
     @property
@@ -124,7 +128,7 @@ class MatLayout:
 def matrix_workspace_bytes(rows: int, cols: int, unit: int) -> int:
     m, n = min(rows, cols), max(rows, cols)
     mp, np_ = _round_up(m, unit), _round_up(n, unit)
-    return (_round_up(mp * (np_ + LD_PAD) * 2, _ALIGN) + 2 * _round_up(np_ * (mp + LD_PAD) * 2, _ALIGN) +
+    return (2 * _round_up(max(mp * (np_ + LD_PAD), np_ * (mp + LD_PAD)) * 2, _ALIGN) +
             3 * _round_up(mp * (mp + LD_PAD) * 2, _ALIGN))
 
 
@@ -224,10 +228,10 @@ class ChunkPlan:
         for index, rows, cols in mats:
             m, n = min(rows, cols), max(rows, cols)
             lay = MatLayout(index, rows, cols, m, n, _round_up(m, T), _round_up(n, T), rows <= cols)
-            xb = _round_up(lay.mp * lay.ldn * 2, _ALIGN)
-            tb = _round_up(lay.np_ * lay.ldm * 2, _ALIGN)
+            # (an m x n buffer also holds the n x m matrix of a run without iterations, in either pitch)
+            xb = _round_up(max(lay.mp * lay.ldn, lay.np_ * lay.ldm) * 2, _ALIGN)
             ab = _round_up(lay.mp * lay.ldm * 2, _ALIGN)
-            for name, nbytes in (("X", xb), ("XT0", tb), ("XT1", tb), ("A", ab), ("B", ab), ("CA", ab)):
+            for name, nbytes in (("X0", xb), ("X1", xb), ("A", ab), ("B", ab), ("CA", ab)):
                 lay.off[name] = off
                 off += nbytes
             self.layouts.append(lay)
@@ -254,7 +258,8 @@ class ChunkPlan:
             off += _round_up(lay.mp * (lay.mp // ROWSUM_SLOT) * 4, _ALIGN) if self.aol else 0
         rowblk = [lay.mp // AOL_ROWS for lay in self.layouts]
         self.aol_row_prefix = np.concatenate([[0], np.cumsum(rowblk)]).astype(np.int32)
-        segblk = [b for lay in self.layouts for b in (lay.mp // AOL_ROWS, lay.np_ // AOL_ROWS, lay.mp // AOL_ROWS)]
+        # segments of the rescaling launch per matrix: rows of X, (rows of X^T: none is kept), rows of A
+        segblk = [b for lay in self.layouts for b in (lay.mp // AOL_ROWS, 0, lay.mp // AOL_ROWS)]
         self.aol_seg_prefix = np.concatenate([[0], np.cumsum(segblk)]).astype(np.int32)
         # job lists: the symmetric products share their tiles but not their reduction length
         # (X X^T reduces over n, the polynomial over m), and only the former is ever split
@@ -307,29 +312,25 @@ class ChunkPlan:
         return np.ascontiguousarray(logical[xcd_permutation(len(logical), group)])
 
     # ---- descriptor tables -----------------------------------------------------------------
-    def result_buffer(self, lay: MatLayout) -> str:
-        if self.steps == 0:
-            return "X" if lay.wide else "XT0"
-        return "X" if lay.wide else ("XT1" if self.steps % 2 else "XT0")
-
     def gemm_descs(self, base: int) -> np.ndarray:
         """[N_PHASES, nmat] MuonGemmDesc table for a workspace at device address `base`."""
         d = np.zeros((N_PHASES, self.nmat), dtype=_lib.GEMM_DESC)
         for k, lay in enumerate(self.layouts):
             p = {name: base + o for name, o in lay.off.items()}
             mp, np_ = lay.mp, lay.np_
-            s = d[PH_SYRK, k]
-            s["P"] = s["Q"] = p["X"]
-            s["ldp"] = s["ldq"] = lay.ldn
-            s["K"] = np_
-            s["C"] = s["CT"] = p["A"]
-            if self.reference_rounding:
-                s["C2"] = s["C2T"] = p["CA"]
-            s["ldc"] = s["ldct"] = lay.ldm
-            s["rows"] = s["colsn"] = mp
-            if self.aol:                # used by the launch that carries MUON_AMD_GEMM_ROWSUM only
-                s["rowsum"] = base + self.off_rowsum[k]
-                s["ld_rowsum"] = mp // ROWSUM_SLOT
+            for ph, src in ((PH_SYRK, "X0"), (PH_SYRK_ODD, "X1")):
+                s = d[ph, k]
+                s["P"] = s["Q"] = p[src]
+                s["ldp"] = s["ldq"] = lay.ldn
+                s["K"] = np_
+                s["C"] = s["CT"] = p["A"]
+                if self.reference_rounding:
+                    s["C2"] = s["C2T"] = p["CA"]
+                s["ldc"] = s["ldct"] = lay.ldm
+                s["rows"] = s["colsn"] = mp
+                if self.aol:                # used by the launch that carries MUON_AMD_GEMM_ROWSUM only
+                    s["rowsum"] = base + self.off_rowsum[k]
+                    s["ld_rowsum"] = mp // ROWSUM_SLOT
             q = d[PH_POLY, k]
             q["P"] = p["CA"] if self.reference_rounding else p["A"]
             q["Q"] = q["D"] = p["A"]
@@ -342,43 +343,42 @@ class ChunkPlan:
             for name in _lib.GEMM_DESC.names:
                 f[name] = q[name]
             f["CT"] = 0
-            for ph, src, dst in ((PH_UPD_EVEN, "XT0", "XT1"), (PH_UPD_ODD, "XT1", "XT0")):
+            # X' = a X + B X: P = B (row-major along k), Q = X itself, k-major; X' goes to the other buffer
+            for ph, src, dst in ((PH_UPD_EVEN, "X0", "X1"), (PH_UPD_ODD, "X1", "X0")):
                 u = d[ph, k]
                 u["P"] = p["B"]
                 u["ldp"] = lay.ldm
-                u["Q"] = p[src]
-                u["ldq"] = lay.ldm
+                u["Q"] = u["D"] = p[src]
+                u["ldq"] = u["ldd"] = lay.ldn
+                u["q_kmajor"] = 1
                 u["K"] = mp
-                u["D"] = u["C"] = p["X"]
-                u["ldd"] = u["ldc"] = lay.ldn
-                u["CT"] = p[dst]
-                u["ldct"] = lay.ldm
+                u["C"] = p[dst]
+                u["ldc"] = lay.ldn
                 u["rows"] = mp
                 u["colsn"] = np_
+            # the last update product carries the parameter step in its epilogue and stores nothing
+            # itself (validate_gemm still wants an output: the buffer it would write is named)
             last = d[PH_UPD_LAST, k]
-            if self.steps > 0:
-                last_src = d[PH_UPD_EVEN if (self.steps - 1) % 2 == 0 else PH_UPD_ODD, k]
-                for name in _lib.GEMM_DESC.names:
-                    last[name] = last_src[name]
-                if lay.wide:
-                    last["CT"] = 0
-                else:
-                    last["C"] = 0
-            else:
-                for name in _lib.GEMM_DESC.names:   # never launched; keep it well formed
-                    last[name] = d[PH_UPD_EVEN, k][name]
+            last_src = d[PH_UPD_EVEN if (max(self.steps, 1) - 1) % 2 == 0 else PH_UPD_ODD, k]
+            for name in _lib.GEMM_DESC.names:
+                last[name] = last_src[name]
         return d
 
     def mat_descs(self, base: int) -> np.ndarray:
-        """MuonMatDesc table with the workspace fields filled; tensor pointers are left zero."""
+        """MuonMatDesc table with the workspace fields filled; tensor pointers are left zero.
+        The normalise launch leaves X0 in the orientation the iteration wants: the parameter's own
+        for a wide matrix (`direct`), its transpose for a tall one (`transp`); the other pointer is
+        null and that orientation is not written.  Without iterations (steps = 0) the normalised
+        matrix is the result and is written in the parameter's orientation either way."""
         d = np.zeros(self.nmat, dtype=_lib.MAT_DESC)
         for k, lay in enumerate(self.layouts):
             p = {name: base + o for name, o in lay.off.items()}
             r = d[k]
-            r["u"] = p["XT1"]
-            r["direct"] = p["X"] if lay.wide else p["XT0"]
-            r["transp"] = p["XT0"] if lay.wide else p["X"]
-            r["result"] = p[self.result_buffer(lay)]
+            r["u"] = p["X1"]
+            as_param = lay.wide or self.steps == 0
+            r["direct"] = p["X0"] if as_param else 0
+            r["transp"] = 0 if as_param else p["X0"]
+            r["result"] = p["X0"] if self.steps == 0 else 0
             r["partials"] = base + self.off_partials
             r["denom"] = base + self.off_denoms + 4 * k
             r["rows"], r["cols"] = lay.rows, lay.cols
@@ -391,12 +391,12 @@ class ChunkPlan:
         return d
 
     def aol_descs(self, base: int) -> np.ndarray:
-        """MuonAolDesc table: after the normalise launch X is in `X` and X^T in `XT0`."""
+        """MuonAolDesc table: after the normalise launch X is in `X0` (no transposed copy: `xc` is null)."""
         d = np.zeros(self.nmat, dtype=_lib.AOL_DESC)
         for k, lay in enumerate(self.layouts):
             r = d[k]
-            r["xr"] = base + lay.off["X"]
-            r["xc"] = base + lay.off["XT0"]
+            r["xr"] = base + lay.off["X0"]
+            r["xc"] = 0
             r["gram"] = base + lay.off["A"]
             r["rvec"] = base + self.off_rvec[k]
             r["rowsum"] = base + self.off_rowsum[k]
@@ -407,7 +407,7 @@ class ChunkPlan:
     def phase_scalars(self, phase: int, iteration: int = 0):
         """(alpha, beta, gamma) of the GEMM epilogue for a phase of an iteration."""
         a, b, c = AOL_COEFFS[iteration] if self.aol else NS_COEFFS
-        if phase == PH_SYRK:
+        if phase in (PH_SYRK, PH_SYRK_ODD):
             return 1.0, 0.0, c
         if phase in (PH_POLY, PH_POLY_FULL):
             return (1.0, b, 0.0) if self.reference_rounding else (c, b, 0.0)

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     lib = _lib.load()
-    assert lib.muon_amd_abi_version() == 2
+    assert lib.muon_amd_abi_version() == 3
     for tc, (tr, tcol) in plan.TILE_DIMS.items():
         assert (lib.muon_amd_gemm_tile_rows(tc), lib.muon_amd_gemm_tile_cols(tc)) == (tr, tcol)
     assert lib.muon_amd_gemm_tile_rows(7) < 0 and b"tile class" in lib.muon_amd_last_error()
@@ -63,12 +63,21 @@ def _check_chunk(lib, c):
     T = c.tile
     assert all(plan.tile_class_for(l.m) == c.tile_class for l in c.layouts)
     g = c.gemm_descs(1 << 20)
-    for ph in range(5):
-        jobs = c.syrk_jobs if ph == plan.PH_SYRK else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
+    syrk_phases = (plan.PH_SYRK, plan.PH_SYRK_ODD)
+    for ph in (plan.PH_SYRK, plan.PH_SYRK_ODD, plan.PH_POLY, plan.PH_UPD_EVEN, plan.PH_UPD_ODD, plan.PH_UPD_LAST):
+        jobs = c.syrk_jobs if ph in syrk_phases else c.sym_jobs if ph == plan.PH_POLY else c.full_jobs
         tile_class = c.update_class if jobs is c.full_jobs else c.tile_class     # the update products may use larger tiles
         rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[ph]), c.nmat, _lib.host_ptr(jobs), len(jobs), tile_class,
-                                        c.split_slots if ph == plan.PH_SYRK else 0)
+                                        c.split_slots if ph in syrk_phases else 0)
         assert rc == 0, lib.muon_amd_last_error()
+    # the update product reads X itself, k-major, and writes the other buffer; X X^T follows the iterate
+    for k, l in enumerate(c.layouts):
+        x0, x1 = (1 << 20) + l.off["X0"], (1 << 20) + l.off["X1"]
+        assert g[plan.PH_SYRK, k]["P"] == g[plan.PH_UPD_EVEN, k]["Q"] == g[plan.PH_UPD_EVEN, k]["D"] == x0
+        assert g[plan.PH_SYRK_ODD, k]["P"] == g[plan.PH_UPD_ODD, k]["Q"] == g[plan.PH_UPD_EVEN, k]["C"] == x1
+        assert g[plan.PH_UPD_ODD, k]["C"] == x0
+        assert all(g[ph, k]["q_kmajor"] == 1 and g[ph, k]["CT"] == 0 for ph in (plan.PH_UPD_EVEN, plan.PH_UPD_ODD, plan.PH_UPD_LAST))
+        assert all(g[ph, k]["q_kmajor"] == 0 for ph in (plan.PH_SYRK, plan.PH_SYRK_ODD, plan.PH_POLY))
     assert c.update_class in (c.tile_class, 1)
     TR, TC = c.tile_rows, c.tile_cols
     UR, UC = plan.TILE_DIMS[c.update_class]
@@ -94,9 +103,10 @@ def _check_chunk(lib, c):
     # workspace regions do not overlap and stay inside the chunk's workspace
     regions = []
     for l in c.layouts:
-        size = {"X": l.mp * l.ldn * 2, "XT0": l.np_ * l.ldm * 2, "XT1": l.np_ * l.ldm * 2,
+        size = {"X0": l.mp * l.ldn * 2, "X1": l.mp * l.ldn * 2,
                 "A": l.mp * l.ldm * 2, "B": l.mp * l.ldm * 2, "CA": l.mp * l.ldm * 2}
-        for name in ("X", "XT0", "XT1", "A", "B", "CA"):
+        assert set(l.off) == set(size)            # two copies of X, no transposed one: 2 m n + 3 m^2
+        for name in size:
             regions.append((l.off[name], l.off[name] + size[name]))
     regions += [(c.off_partials, c.off_partials + 4 * c.nblocks), (c.off_denoms, c.off_denoms + 4 * c.nmat)]
     regions.sort()
@@ -137,6 +147,8 @@ def test_random_parameter_lists_plan_into_valid_tables():
     for case in range(60):
         shapes = [(dim(), dim()) for _ in range(rng.randint(1, 12))]
         variant = rng.choice(["ns5", "ns5", "aol4", "aol4_rows"])
+        if variant == "aol4_rows":      # refused below a side of 32
+            shapes = [(max(r, plan.AOL_ROWS_MIN_SIDE), max(c, plan.AOL_ROWS_MIN_SIDE)) for r, c in shapes]
         aol = variant != "ns5"
         biggest = max(plan.matrix_workspace_bytes(r, c, plan.pad_unit(plan.tile_class_for(min(r, c)))) +
                       plan.matrix_scratch_bytes(r, c, plan.tile_class_for(min(r, c)), aol) for r, c in shapes)
@@ -206,7 +218,7 @@ def test_split_reduction_plan():
     assert lib.muon_amd_validate_gemm(*args, _lib.host_ptr(twice), len(twice), c.tile_class, c.split_slots) == -1
 
 
-def test_xcd_permutation_and_result_buffer():
+def test_xcd_permutation_and_orientation_of_the_iterate():
     for n in (1, 7, 8, 9, 136, 1000, 4352):
         for group in (32, 64):
             p = plan.xcd_permutation(n, group)
@@ -214,9 +226,19 @@ def test_xcd_permutation_and_result_buffer():
     p = plan.xcd_permutation(512, 32)            # block b runs on XCD b % 8, slot b // 8
     assert p[:8].tolist() == [0, 32, 64, 96, 128, 160, 192, 224] and p[8] == 1      # a 32-job group per XCD
     assert p[256:264].tolist() == [256, 288, 320, 352, 384, 416, 448, 480]           # next round of groups
-    for steps, want_tall in ((0, "XT0"), (1, "XT1"), (2, "XT0"), (5, "XT1")):
+    # the normalise launch writes X0 in one orientation: the parameter's for a wide matrix and for a run
+    # without iterations (where it is the result), the transposed one for a tall matrix that iterates
+    for steps in (0, 1, 2, 5):
         c = plan.ChunkPlan([(0, 300, 100), (1, 100, 300)], 0, steps, True)
-        assert c.result_buffer(c.layouts[0]) == want_tall and c.result_buffer(c.layouts[1]) == "X"
+        md = c.mat_descs(1 << 20)
+        x0 = [(1 << 20) + l.off["X0"] for l in c.layouts]
+        tall, wide = md[0], md[1]
+        assert wide["direct"] == x0[1] and wide["transp"] == 0
+        assert (tall["direct"], tall["transp"]) == ((x0[0], 0) if steps == 0 else (0, x0[0]))
+        assert all(m["result"] == (m["direct"] if steps == 0 else 0) for m in md)
+        assert all(m["u"] == (1 << 20) + l.off["X1"] for m, l in zip(md, c.layouts))
+    # workspace per matrix: 2 m n + 3 m^2 bf16 elements (padded)
+    assert plan.matrix_workspace_bytes(4096, 14336, 256) == 2 * (2 * 4096 * 14336 + 3 * 4096 * 4096)
 
 
 def test_chunking_respects_the_workspace_cap():
@@ -327,7 +349,8 @@ def test_aol_variant_plan_validates():
     assert lib.muon_amd_aol_rows_per_block() == plan.AOL_ROWS
     assert _lib.AOL_DESC.itemsize == lib.muon_amd_sizeof_aol_desc() == 64
     for variant in ("aol4", "aol4_rows"):
-        chunks = plan.plan_chunks(SHAPES, 5, True, 1 << 30, variant)
+        shapes = [sh for sh in SHAPES if variant == "aol4" or min(sh) >= plan.AOL_ROWS_MIN_SIDE]
+        chunks = plan.plan_chunks(shapes, 5, True, 1 << 30, variant)
         for c in chunks:
             assert c.variant == variant and c.aol and c.steps == len(plan.AOL_COEFFS) == 4 and not c.reference_rounding
             d = c.aol_descs(1 << 20)

@@ -23,7 +23,7 @@ def _syrk_both_ways(lib, shapes, seed):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
     for lay in chunk.layouts:       # the operand: X, zero padded, rows of pitch ldn
-        x = ws[lay.off["X"]: lay.off["X"] + lay.mp * lay.ldn * 2].view(torch.bfloat16).view(lay.mp, lay.ldn)
+        x = ws[lay.off["X0"]: lay.off["X0"] + lay.mp * lay.ldn * 2].view(torch.bfloat16).view(lay.mp, lay.ldn)
         x[:lay.m, :lay.n] = (torch.randn(lay.m, lay.n, device="cuda", generator=gen) * 0.05).bfloat16()
     gemm = chunk.gemm_descs(base)[plan.PH_SYRK]
     jobs = chunk.syrk_jobs
@@ -60,7 +60,7 @@ def _syrk_both_ways(lib, shapes, seed):
         assert torch.equal(w, g)
     # and the product is the right one (fp32 matmul of the same bf16 operand)
     lay = chunk.layouts[0]
-    x = ws[lay.off["X"]: lay.off["X"] + lay.mp * lay.ldn * 2].view(torch.bfloat16).view(lay.mp, lay.ldn)[:lay.m, :lay.n].float()
+    x = ws[lay.off["X0"]: lay.off["X0"] + lay.mp * lay.ldn * 2].view(torch.bfloat16).view(lay.mp, lay.ldn)[:lay.m, :lay.n].float()
     a = got[0].view(torch.bfloat16).view(lay.mp, lay.ldm)[:lay.m, :lay.m].float()
     ref = x @ x.T
     assert float((a - ref).norm() / ref.norm()) < 5e-3
