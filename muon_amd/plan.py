@@ -67,10 +67,12 @@ def tile_class_for(m: int) -> int:
 
 
 GEMM_BK = 64                            # k-block of the GEMM kernel: K and every job's K range are multiples
-SPLIT_MAX_M = 512                       # X X^T of a matrix this short ...
-SPLIT_MIN_KBLOCKS = 32                  # ... and at least this long (in k-blocks) is split ...
-SPLIT_KBLOCKS_PER_JOB = 16              # ... into jobs of about this many k-blocks, at most SPLIT_MAX
-SPLIT_MAX = 16
+# (measurement knob: MUON_AMD_SPLIT = "max_m,min_kblocks,kblocks_per_job,max")
+_SPLIT = [int(v) for v in os.environ.get("MUON_AMD_SPLIT", "512,32,24,16").split(",")]
+SPLIT_MAX_M = _SPLIT[0]                 # X X^T of a matrix this short ...
+SPLIT_MIN_KBLOCKS = _SPLIT[1]           # ... and at least this long (in k-blocks) is split ...
+SPLIT_KBLOCKS_PER_JOB = _SPLIT[2]       # ... into jobs of about this many k-blocks, at most SPLIT_MAX
+SPLIT_MAX = _SPLIT[3]
 
 
 def split_factor(mp: int, kdim: int) -> int:
