@@ -187,10 +187,10 @@ def test_split_reduction_plan():
     """X X^T of a short, very wide matrix is split along K by a rule that looks at the matrix alone."""
     lib = _lib.load()
     assert [plan.split_factor(128, 16384), plan.split_factor(512, 4608), plan.split_factor(512, 2304),
-            plan.split_factor(256, 576), plan.split_factor(768, 3072), plan.split_factor(4096, 14336)] == [16, 4, 2, 1, 1, 1]
+            plan.split_factor(256, 576), plan.split_factor(768, 3072), plan.split_factor(4096, 14336)] == [10, 3, 1, 1, 1, 1]
     c = plan.plan_chunks([(128, 16384), (16384, 128), (512, 4608), (64, 216)], 5, True, 1 << 30)[0]
     g = c.gemm_descs(1 << 20)
-    assert c.split_slots == 16 + 16 + 10 * 4 and len(c.syrk_jobs) == c.split_slots + 1
+    assert c.split_slots == 10 + 10 + 10 * 3 and len(c.syrk_jobs) == c.split_slots + 1
     assert np.all(c.sym_jobs["split"] == 0) and np.all(c.full_jobs["split"] == 0)      # only X X^T is split
     rc = lib.muon_amd_validate_gemm(_lib.host_ptr(g[plan.PH_SYRK]), c.nmat, _lib.host_ptr(c.syrk_jobs),
                                     len(c.syrk_jobs), c.tile_class, c.split_slots)
