@@ -453,6 +453,26 @@ def test_update_products_take_large_tiles_only_where_they_fill_the_gpu():
     assert c.tile_class == 1 and c.update_class == 1
 
 
+def test_jobs_of_unequal_length_are_dealt_so_that_the_cus_stay_balanced():
+    """A launch whose matrices differ in shape has jobs of different lengths; the planner deals them to
+    the XCDs in half or quarter super-blocks when whole ones would leave some CUs with much more work."""
+    gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    (c,) = plan.plan_chunks(gpt2, 5, True, 16 << 30)
+    kb = (c.syrk_jobs["k1"] - c.syrk_jobs["k0"]) // plan.GEMM_BK
+    assert sorted(set(kb.tolist())) == [12, 36, 48] and len(kb) == 48 * 21
+    cu, xcd = plan.launch_imbalance(kb, 0)
+    assert cu < 1.03 and xcd < 1.02                       # (whole super-blocks: 1.14 and 1.10)
+    logical = np.sort(kb)[::-1]                           # the list order: same-shape matrices adjacent
+    whole = plan.launch_imbalance(logical[plan.xcd_permutation(len(kb), 64)], 0)
+    assert whole[0] > 1.12 and plan.choose_xcd_group(logical, 0, 64) in (16, 32)
+    # jobs of equal length: nothing to gain, the super-block stays whole
+    assert plan.choose_xcd_group(np.full(1008, 12), 0, 64) == 64
+    assert plan.choose_xcd_group(np.full(4352, 64), 1, 32) == 32
+    # every job still appears exactly once
+    assert sorted(zip(c.syrk_jobs["desc"].tolist(), c.syrk_jobs["i0"].tolist(), c.syrk_jobs["j0"].tolist())) == \
+        sorted((d, i, j) for d in range(48) for i in range(0, 768, 128) for j in range(i, 768, 128))
+
+
 def test_rows_only_aol_is_refused_below_its_stated_size():
     """plan_chunks refuses the rows-only AOL rescaling for a matrix with a side below
     AOL_ROWS_MIN_SIDE (the map does not contract there), and only that variant."""
