@@ -203,10 +203,21 @@ def xcd_permutation(njobs: int, group: int = 32) -> np.ndarray:
         seg = -(-njobs // N_XCD)
         idx = np.arange(N_XCD * seg, dtype=np.int64).reshape(N_XCD, seg).T.reshape(-1)
         return idx[idx < njobs]
-    b = np.arange(-(-njobs // (N_XCD * group)) * N_XCD * group, dtype=np.int64)
+    full = njobs // (N_XCD * group) * (N_XCD * group)
+    perm = np.empty(njobs, dtype=np.int64)
+    b = np.arange(full, dtype=np.int64)
     x, s = b % N_XCD, b // N_XCD
-    idx = ((s // group) * N_XCD + x) * group + (s % group)
-    return idx[idx < njobs]
+    perm[:full] = ((s // group) * N_XCD + x) * group + (s % group)
+    # What is left over after the last whole set of eight groups still goes to the XCDs in contiguous
+    # runs: block full + 8 i + x is slot i of XCD x, which takes the i-th job of its run.  (Dealing
+    # whole groups and dropping the missing jobs would shift every later block to another XCD.)
+    rem = njobs - full
+    if rem:
+        count = (rem - np.arange(N_XCD) + N_XCD - 1) // N_XCD       # blocks XCD x has in the remainder
+        start = full + np.concatenate([[0], np.cumsum(count)[:-1]])
+        t = np.arange(rem, dtype=np.int64)
+        perm[full:] = start[t % N_XCD] + t // N_XCD
+    return perm
 
 
 # Cost of a job in k-blocks for balancing a launch: its reduction plus what its prologue and

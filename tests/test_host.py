@@ -223,6 +223,16 @@ def test_xcd_permutation_and_orientation_of_the_iterate():
         for group in (32, 64):
             p = plan.xcd_permutation(n, group)
             assert sorted(p.tolist()) == list(range(n))
+    # a job count that is no multiple of eight groups: what is left over still reaches every XCD as
+    # one contiguous run of the list (block b is on XCD b % 8), no XCD gets more than one job more than
+    # another, and nothing shifts the whole groups before it
+    for n, group in ((966, 64), (1296, 32), (454, 64), (1000, 16)):
+        p = plan.xcd_permutation(n, group)
+        full = n // (8 * group) * (8 * group)
+        assert p[:full].tolist() == plan.xcd_permutation(full, group).tolist()
+        runs = [p[full:][x::8] for x in range(8)]
+        assert all(len(r) == 0 or r.tolist() == list(range(r[0], r[0] + len(r))) for r in runs)
+        assert max(map(len, runs)) - min(map(len, runs)) <= 1
     p = plan.xcd_permutation(512, 32)            # block b runs on XCD b % 8, slot b // 8
     assert p[:8].tolist() == [0, 32, 64, 96, 128, 160, 192, 224] and p[8] == 1      # a 32-job group per XCD
     assert p[256:264].tolist() == [256, 288, 320, 352, 384, 416, 448, 480]           # next round of groups
