@@ -482,21 +482,87 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
     order = sorted(range(len(shapes)),
                    key=lambda i: (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]),
                                   -shapes[i][0], i))
-    chunks, cur, cur_bytes, cur_class = [], [], 0, None
-    for i in order:
-        rows, cols = shapes[i]
-        tc = tile_class_for(min(rows, cols))
-        need = (matrix_workspace_bytes(rows, cols, pad_unit(tc)) +
-                matrix_scratch_bytes(rows, cols, tc, variant in ("aol4", "aol4_rows")))
-        if cur and (tc != cur_class or cur_bytes + need > workspace_cap):
-            chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding, variant))
-            cur, cur_bytes = [], 0
-        cur.append((i, rows, cols))
-        cur_bytes += need
-        cur_class = tc
-    if cur:
-        chunks.append(ChunkPlan(cur, cur_class, steps, reference_rounding, variant))
+    need = [matrix_workspace_bytes(*shapes[i], pad_unit(tile_class_for(min(shapes[i])))) +
+            matrix_scratch_bytes(*shapes[i], tile_class_for(min(shapes[i])), variant in ("aol4", "aol4_rows"))
+            for i in order]
+    chunks, pos = [], 0
+    while pos < len(order):
+        tc = tile_class_for(min(shapes[order[pos]]))
+        end = pos                                          # the run of this tile class in the list
+        while end < len(order) and tile_class_for(min(shapes[order[end]])) == tc:
+            end += 1
+        kmax, nbytes = 0, 0                                # as many of it as stay under the cap ...
+        while pos + kmax < end and (kmax == 0 or nbytes + need[pos + kmax] <= workspace_cap):
+            nbytes += need[pos + kmax]
+            kmax += 1
+        # ... cut where the launches of this chunk and of what it leaves behind fill their last rounds best
+        k = kmax
+        if TAIL_AWARE_CHUNKS and pos + kmax < end:         # (a run that fits one chunk stays whole)
+            k = _best_cut([shapes[i] for i in order[pos:end]], need[pos:end], tc, kmax, workspace_cap)
+        chunks.append(ChunkPlan([(i, *shapes[i]) for i in order[pos:pos + k]], tc, steps, reference_rounding, variant))
+        pos += k
     return chunks
+
+
+TAIL_AWARE_CHUNKS = os.environ.get("MUON_AMD_TAIL_AWARE_CHUNKS", "1") != "0"      # measurement knob
+KBLOCK_US = {0: 0.645, 1: 1.58}         # a CU's time per k-block of its tiles (two co-resident 128 x 128 tiles share it)
+CHUNK_FIXED_US = 200.0                  # what one more chunk costs: 18 more launches that fill and drain the GPU
+
+
+def _chunk_time_us(mats, tile_class: int) -> tuple[float, float]:
+    """(estimated, ideal) time of the fifteen GEMM launches of one iteration-set of a chunk holding
+    `mats` [(rows, cols)], from the busiest CU of every launch (jobs in list order, job j on
+    workgroup j % grid; see launch_imbalance).  The ideal has every CU equally busy."""
+    unit = pad_unit(tile_class)
+    dims = [(_round_up(min(r, c), unit), _round_up(max(r, c), unit)) for r, c in mats]
+    big = (tile_class == 1 or
+           (UPDATE_CLASS != "0" and all(mp % 256 == 0 and np_ % 256 == 0 for mp, np_ in dims) and
+            (UPDATE_CLASS == "1" or sum((mp // 256) * (np_ // 256) for mp, np_ in dims) >= RESIDENT_BIG_TILE_WORKGROUPS)))
+    est = ideal = 0.0
+    T = TILE_DIMS[tile_class][0]
+    for kind in ("syrk", "poly", "update"):
+        tc = (1 if big else 0) if kind == "update" else tile_class
+        TT = TILE_DIMS[tc][0] if kind == "update" else T
+        counts, costs = [], []
+        for mp, np_ in dims:
+            mt = mp // TT
+            if kind == "update":
+                counts.append(mt * (np_ // TT)); costs.append(mp // GEMM_BK)
+            else:
+                kb = (np_ if kind == "syrk" else mp) // GEMM_BK
+                ns = split_factor(mp, np_) if kind == "syrk" else 1
+                counts.append(mt * (mt + 1) // 2 * ns); costs.append(kb // ns)
+        cost = np.repeat(np.asarray(costs, dtype=np.float64) + JOB_FIXED_KBLOCKS[tc], counts)
+        grid = min(len(cost), N_CU * WORKGROUPS_PER_CU[tc])
+        cu = np.bincount((np.arange(len(cost)) % grid) % N_CU, weights=cost, minlength=N_CU)
+        est += cu.max() * KBLOCK_US[tc]
+        ideal += cost.sum() / N_CU * KBLOCK_US[tc]
+    return est, ideal
+
+
+def _best_cut(mats, nbytes, tile_class: int, kmax: int, cap: int) -> int:
+    """How many of the first kmax matrices of the run `mats` (one tile class, in list order; `nbytes`
+    their workspace needs) the next chunk takes: the count, between half of kmax and kmax, that makes
+    the whole run cheapest.  A chunk costs what the busiest CU of each of its launches takes plus the
+    launches themselves; what it leaves behind is charged as the chunk it would make if it fits one,
+    else at 3 % over its ideal time plus the chunks its bytes need.  So a cut moves to where the
+    launches fill their last rounds (51 matrices of 4096 x 14336 are 27.09 rounds of X X^T tiles on 256
+    CUs, 47 of them 24.97), but never splits off a handful of matrices into launches of their own."""
+    if kmax <= 2:
+        return kmax
+    fixed = CHUNK_FIXED_US / 5                             # per iteration, like the launch times
+    best, best_cost = kmax, None
+    for k in range(kmax, max(kmax // 2, 1) - 1, -1):
+        est, _ = _chunk_time_us(mats[:k], tile_class)
+        cost = est + fixed
+        rest = mats[k:]
+        if rest:
+            rest_bytes = sum(nbytes[k:])
+            r_est, r_ideal = _chunk_time_us(rest, tile_class)
+            cost += (r_est + fixed) if rest_bytes <= cap else (r_ideal * 1.03 + fixed * rest_bytes / cap)
+        if best_cost is None or cost < best_cost * 0.997:     # ties go to the larger chunk
+            best, best_cost = k, cost
+    return best
 
 
 def adam_block_prefix(numels) -> np.ndarray:

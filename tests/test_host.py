@@ -483,6 +483,30 @@ def test_jobs_of_unequal_length_are_dealt_so_that_the_cus_stay_balanced():
         sorted((d, i, j) for d in range(48) for i in range(0, 768, 128) for j in range(i, 768, 128))
 
 
+def test_chunk_cuts_move_to_where_the_launches_fill_their_last_rounds():
+    """When the workspace cap forces a cut inside a run of matrices, the cut goes where the launches of
+    the chunk (and of what it leaves behind) waste least on partial last rounds; a run that fits one
+    chunk is never split, and every matrix still lands in exactly one chunk, in list order."""
+    llama = [(4096, 4096)] * 64 + [(1024, 4096)] * 64 + [(14336, 4096)] * 64 + [(4096, 14336)] * 32
+    chunks = plan.plan_chunks(llama, 5, True, 16 << 30)
+    assert [len(c.layouts) for c in chunks] == [50, 47, 127]
+    assert all(c.workspace_bytes <= (16 << 30) for c in chunks)
+    assert sorted(l.index for c in chunks for l in c.layouts) == list(range(len(llama)))
+    # 47 matrices of m = 4096: 47 * 136 symmetric tiles = 24.97 rounds of 256 workgroups
+    assert len(chunks[1].syrk_jobs) == 47 * 136 and 47 * 136 / 256 > 24.9
+    for cap in (4 << 30, 8 << 30, 12 << 30):
+        cs = plan.plan_chunks(llama, 5, True, cap)
+        assert all(c.workspace_bytes <= cap for c in cs)
+        assert sorted(l.index for c in cs for l in c.layouts) == list(range(len(llama)))
+    # est >= ideal, equal jobs on a multiple of the grid are ideal
+    est, ideal = plan._chunk_time_us([(4096, 4096)] * 32, 1)
+    assert abs(est - ideal) < 1e-6 * ideal
+    est, ideal = plan._chunk_time_us([(4096, 4096)] * 33, 1)
+    assert est > 1.01 * ideal
+    (c,) = plan.plan_chunks([(768, 3072)] * 46 + [(768, 768)] * 2, 5, True, 16 << 30)      # fits: stays whole
+    assert len(c.layouts) == 48
+
+
 def test_rows_only_aol_is_refused_below_its_stated_size():
     """plan_chunks refuses the rows-only AOL rescaling for a matrix with a side below
     AOL_ROWS_MIN_SIDE (the map does not contract there), and only that variant."""
