@@ -2,7 +2,9 @@
 104-109, 265-291), executed by the gfx950 kernels of libmuon_amd.so."""
 from __future__ import annotations
 
+import threading
 from collections import OrderedDict
+from contextlib import contextmanager
 
 import torch
 
@@ -15,21 +17,47 @@ _ENGINE_CACHE: "OrderedDict[tuple, object]" = OrderedDict()
 _ENGINE_CACHE_MAX = 4     # each cached engine holds its bf16 workspace
 
 
+_CACHE_LOCK = threading.Lock()
+
+
 def _cached(key, make):
-    eng = _ENGINE_CACHE.get(key)
-    if eng is None:
-        eng = make()
-        _ENGINE_CACHE[key] = eng
-        while len(_ENGINE_CACHE) > _ENGINE_CACHE_MAX:
-            _ENGINE_CACHE.popitem(last=False)
-    else:
-        _ENGINE_CACHE.move_to_end(key)
-    return eng
+    with _CACHE_LOCK:
+        eng = _ENGINE_CACHE.get(key)
+        if eng is None:
+            eng = make()
+            eng._fn_lock = threading.Lock()       # one caller at a time enqueues on this engine
+            eng._fn_done = None                   # event after the launches of its last call
+            _ENGINE_CACHE[key] = eng
+            while len(_ENGINE_CACHE) > _ENGINE_CACHE_MAX:
+                _ENGINE_CACHE.popitem(last=False)
+        else:
+            _ENGINE_CACHE.move_to_end(key)
+        return eng
+
+
+@contextmanager
+def _exclusive(eng, device):
+    """A cached engine owns one workspace, so its calls must not overlap, neither on the host (two
+    threads enqueueing at once) nor on the device (two streams running its launches side by side):
+    callers take the engine's lock, and the stream of a call waits for the launches of the call
+    before it.  (Not while a HIP graph is being captured: the event of an earlier, uncaptured call
+    cannot be waited for there, and a capture runs on one stream anyway.)"""
+    with eng._fn_lock:
+        stream = torch.cuda.current_stream(device)
+        capturing = torch.cuda.is_current_stream_capturing()
+        if eng._fn_done is not None and not capturing:
+            stream.wait_event(eng._fn_done)
+        yield
+        if not capturing:
+            done = torch.cuda.Event()
+            done.record(stream)
+            eng._fn_done = done
 
 
 def clear_engine_cache() -> None:
     """Drop the workspaces cached by the functional entry points."""
-    _ENGINE_CACHE.clear()
+    with _CACHE_LOCK:
+        _ENGINE_CACHE.clear()
 
 
 def _rounding_flag(rounding: str) -> bool:
@@ -61,10 +89,11 @@ def _orthogonalise(G: torch.Tensor, steps: int, epsilon: float, ref: bool, varia
         eng = _cached(("ns", G.device, rows, cols, batch, int(steps), ref, variant),
                       lambda: MuonGroupEngine([(rows, cols)] * batch, G.device, int(steps), ref, variant=variant))
         gsz, osz = rows * cols * G.element_size(), rows * cols * 2
-        eng.run([G.data_ptr() + b * gsz for b in range(batch)], [0] * batch, [0] * batch,
-                [out.data_ptr() + b * osz for b in range(batch)], [1.0] * batch,
-                [_src_dtype(G)] * batch, beta=0.0, nesterov=False, mutate_grad=False,
-                eps=float(epsilon), lr=0.0, weight_decay=0.0)
+        with _exclusive(eng, G.device):
+            eng.run([G.data_ptr() + b * gsz for b in range(batch)], [0] * batch, [0] * batch,
+                    [out.data_ptr() + b * osz for b in range(batch)], [1.0] * batch,
+                    [_src_dtype(G)] * batch, beta=0.0, nesterov=False, mutate_grad=False,
+                    eps=float(epsilon), lr=0.0, weight_decay=0.0)
     return out
 
 
@@ -127,11 +156,12 @@ def muon_update(grad: torch.Tensor, momentum: torch.Tensor, beta: float = 0.95,
                       lambda: MuonGroupEngine([(rows, cols)] * batch, grad.device, int(ns_steps), ref,
                                               variant=ns_variant))
         gsz, osz = rows * cols * grad.element_size(), rows * cols * 2
-        eng.run([grad.data_ptr() + b * gsz for b in range(batch)],
-                [momentum.data_ptr() + b * gsz for b in range(batch)], [0] * batch,
-                [out.data_ptr() + b * osz for b in range(batch)], [scale] * batch,
-                [_src_dtype(grad)] * batch, beta=beta, nesterov=bool(nesterov), mutate_grad=True,
-                eps=1e-7, lr=0.0, weight_decay=0.0)
+        with _exclusive(eng, grad.device):
+            eng.run([grad.data_ptr() + b * gsz for b in range(batch)],
+                    [momentum.data_ptr() + b * gsz for b in range(batch)], [0] * batch,
+                    [out.data_ptr() + b * osz for b in range(batch)], [scale] * batch,
+                    [_src_dtype(grad)] * batch, beta=beta, nesterov=bool(nesterov), mutate_grad=True,
+                    eps=1e-7, lr=0.0, weight_decay=0.0)
     return out
 
 
@@ -150,6 +180,7 @@ def adam_update(grad, buf1, buf2, step, betas, eps) -> torch.Tensor:
         return out
     with torch.cuda.device(grad.device):
         eng = _cached(("adam", grad.device, grad.numel()), lambda: AdamGroupEngine([grad.numel()], grad.device))
-        eng.run([0], [grad.data_ptr()], [buf1.data_ptr()], [buf2.data_ptr()], [out.data_ptr()],
-                lr=0.0, weight_decay=0.0, betas=betas, eps=float(eps), step=step, dtypes=[_src_dtype(grad)])
+        with _exclusive(eng, grad.device):
+            eng.run([0], [grad.data_ptr()], [buf1.data_ptr()], [buf2.data_ptr()], [out.data_ptr()],
+                    lr=0.0, weight_decay=0.0, betas=betas, eps=float(eps), step=step, dtypes=[_src_dtype(grad)])
     return out

@@ -211,6 +211,41 @@ def test_tensor_hyper_parameters_and_side_streams_change_nothing(M):
             assert torch.equal(a.detach(), b.detach()), (step, tuple(a.shape))
 
 
+def test_functional_calls_from_several_threads_and_streams_share_an_engine_safely(M):
+    """The functional entry points cache one engine (one workspace) per shape.  Calls of the same
+    shape from several threads, each on a stream of its own, must not run side by side in that
+    workspace: every result equals the one computed alone."""
+    import threading
+    torch.manual_seed(11)
+    M.clear_engine_cache()
+    inputs = [torch.randn(256, 512, device="cuda") * 0.02 for _ in range(8)]
+    want = [M.zeropower_via_newtonschulz5(g).clone() for g in inputs]
+    torch.cuda.synchronize()
+    got, errors = [None] * len(inputs), []
+
+    def work(lo, hi):
+        try:
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.default_stream())
+            with torch.cuda.stream(s):
+                for rep in range(3):
+                    for i in range(lo, hi):
+                        got[i] = M.zeropower_via_newtonschulz5(inputs[i])
+            s.synchronize()
+        except Exception as e:          # surfaces in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(k * 2, k * 2 + 2)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for w, g in zip(want, got):
+        assert torch.equal(w, g)
+
+
 def test_usual_training_loop_companions(M):
     """A learning-rate scheduler, gradient clipping and a gradient scaler around the optimizer, as a
     training script has them: the scheduler's `initial_lr` key in the groups, its wrapped step(),
