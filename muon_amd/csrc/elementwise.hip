@@ -471,17 +471,33 @@ __device__ __forceinline__ void adam_block(const MuonAdamDesc& d, int64_t block_
                 if (upd) Stored<T>::st4(upd + e, uu);
             }
         } else {
+            // The last, partial pass of a tensor (or a tensor at an odd address): element accesses, four
+            // elements at a time with their loads ahead of the arithmetic.  The loop stays rolled: a
+            // launch over a few small tensors runs this code once per wave, and what it then waits for
+            // is the instruction fetch (unrolled, the pass is several thousand instructions long).
+#pragma unroll 1
             for (int it = 0; it < EW_ITERS; ++it) {
                 const int64_t e0 = base + (it * EW_THREADS + threadIdx.x) * EW_VEC;
+                if (e0 >= numel) break;
+                float gs[EW_VEC], ms[EW_VEC], vs[EW_VEC], ps[EW_VEC];
 #pragma unroll
                 for (int k = 0; k < EW_VEC; ++k) {
                     const int64_t e = e0 + k;
-                    if (e >= numel) break;
-                    float mm = Stored<T>::ld(m + e), v2 = Stored<T>::ld(v + e);
-                    const float uu = adam_one<T>(Stored<T>::ld(g + e), &mm, &v2, w1, w2, eps, bias1, bias2);
+                    const bool in = e < numel;
+                    gs[k] = in ? Stored<T>::ld(g + e) : 0.f;
+                    ms[k] = in ? Stored<T>::ld(m + e) : 0.f;
+                    vs[k] = in ? Stored<T>::ld(v + e) : 0.f;
+                    ps[k] = (in && p) ? Stored<T>::ld(p + e) : 0.f;
+                }
+#pragma unroll
+                for (int k = 0; k < EW_VEC; ++k) {
+                    const int64_t e = e0 + k;
+                    if (e >= numel) continue;
+                    float mm = ms[k], v2 = vs[k];
+                    const float uu = adam_one<T>(gs[k], &mm, &v2, w1, w2, eps, bias1, bias2);
                     Stored<T>::st(m + e, mm);
                     Stored<T>::st(v + e, v2);
-                    if (p) Stored<T>::st(p + e, apply_one<T>(Stored<T>::ld(p + e), uu, neg_lr, wd_factor));
+                    if (p) Stored<T>::st(p + e, apply_one<T>(ps[k], uu, neg_lr, wd_factor));
                     if (upd) Stored<T>::st(upd + e, uu);
                 }
             }
