@@ -266,28 +266,40 @@ __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __res
     const bool vec_ok = (d.cols % 8 == 0) && aligned_to(u, 16);
 
     constexpr int CH = NT_TILE / 8;                      // 8-element chunks per tile row
+    constexpr int NI = NT_TILE * CH / 256;               // chunks per thread
+    // every load of the tile goes out before the first result is stored (the stores may alias the
+    // loads as far as the compiler knows, so interleaved each load would wait for the store before it)
+    u32x4e raws[NI];
 #pragma unroll
-    for (int i = 0; i < NT_TILE * CH / 256; ++i) {
+    for (int i = 0; i < NI; ++i) {
+        const int q = threadIdx.x + i * 256;
+        const int gr = R0 + q / CH, gc = C0 + (q % CH) * 8;
+        raws[i] = u32x4e{0u, 0u, 0u, 0u};
+        if (gr < d.rows) {
+            const int64_t off = static_cast<int64_t>(gr) * d.cols + gc;
+            if (vec_ok && gc + 8 <= d.cols) {
+                raws[i] = gld4u(u + off);
+            } else {
+                uint16_t t[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) t[k] = (gc + k < d.cols) ? u[off + k] : static_cast<uint16_t>(0);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) raws[i][k] = t[2 * k] | (static_cast<uint32_t>(t[2 * k + 1]) << 16);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
         const int q = threadIdx.x + i * 256;
         const int r = q / CH, cc = (q % CH) * 8;
         const int gr = R0 + r, gc = C0 + cc;
         uint16_t v[8];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = 0;
+        for (int k = 0; k < 4; ++k) {
+            v[2 * k] = static_cast<uint16_t>(raws[i][k] & 0xffffu);
+            v[2 * k + 1] = static_cast<uint16_t>(raws[i][k] >> 16);
+        }
         if (gr < d.rows) {
-            const int64_t off = static_cast<int64_t>(gr) * d.cols + gc;
-            if (vec_ok && gc + 8 <= d.cols) {
-                const u32x4e raw = gld4u(u + off);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    v[2 * k] = static_cast<uint16_t>(raw[k] & 0xffffu);
-                    v[2 * k + 1] = static_cast<uint16_t>(raw[k] >> 16);
-                }
-            } else {
-#pragma unroll
-                for (int k = 0; k < 8; ++k)
-                    if (gc + k < d.cols) v[k] = u[off + k];
-            }
 #pragma unroll
             for (int k = 0; k < 8; ++k)
                 if (gc + k < d.cols) v[k] = f2bf(bf2f(v[k]) / den);
