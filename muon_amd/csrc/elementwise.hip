@@ -247,9 +247,10 @@ __device__ __forceinline__ void gst4u(uint16_t* p, u32x4e v) {     // read again
     *(__attribute__((address_space(1))) u32x4e*)(p) = v;
 }
 
-// One NT_TILE x NT_TILE tile per block (256-byte row segments in both orientations).  The tile goes through LDS as 32-bit words (two columns each): a
-// thread that later reads word c of rows r .. r+7 holds 8 consecutive elements of the two
-// transposed rows 2c and 2c+1.
+// One NT_TILE x NT_TILE tile per block (256-byte row segments in either orientation; one of the two
+// is written: the parameter's own for a wide matrix, the transposed one for a tall matrix).  The
+// tile goes through LDS as 32-bit words (two columns each): a thread that later reads word c of
+// rows r .. r+7 holds 8 consecutive elements of the two transposed rows 2c and 2c+1.
 __global__ __launch_bounds__(256) void normalize_kernel(const MuonMatDesc* __restrict__ descs,
                                                          const int32_t* __restrict__ prefix,
                                                          int nmat) {

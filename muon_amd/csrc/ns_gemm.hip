@@ -1,30 +1,32 @@
 // Grouped bf16 MFMA GEMM for the Newton-Schulz iteration on gfx950 (CDNA4).
 //
-// Every product of the iteration (muon.py:285-287) is computed as an "NT" GEMM
-//     acc[i][j] = sum_k P[i][k] * Q[j][k]
-// whose two operands are both contiguous along k:
+// Every product of the iteration (muon.py:285-287) is computed by one kernel as
+//     acc[i][j] = sum_k P[i][k] * Q[j][k]          (both operands row-major along k), or
+//     acc[i][j] = sum_k P[i][k] * Q[k][j]          (second operand k-major):
 //     A  = X X^T                P = Q = X            (rows of X)
 //     A A (A symmetric)         P = A or c*A, Q = A  ((A A)[i][j] = sum_k A[i][k] A[j][k])
-//     B X (B symmetric)         P = B, Q = X^T       (X^T kept beside X by the epilogue)
-// so one kernel serves all three, and no operand ever needs a transposing load.  The epilogue
-// fuses the polynomial terms (b*A + c*A*A, a*X + B*X), writes the tile and its transpose (the
-// mirror half of a symmetric result, or X^T for the next iteration), and optionally a scaled
-// copy (c*A).  Symmetric results only compute tiles on or above the diagonal.
+//     B X                       P = B, Q = X itself, k-major (no transposed copy of X is kept:
+//                               the fragments of Q come out of LDS through transposing reads)
+// The epilogue fuses the polynomial terms (b*A + c*A*A, a*X + B*X), writes the tile and, for a
+// symmetric result, its mirror image, and optionally a scaled copy (c*A).  Symmetric results only
+// compute tiles on or above the diagonal.  The update writes X' into a second buffer (every tile of
+// a column block reads all rows of X, so X cannot be overwritten in place).
 //
 // A launch covers a job list of output tiles drawn from many matrices; a workgroup computes one
-// BM x BN tile:
-//   * global_load_lds_dwordx4 streams the operand tiles straight into an LDS ring (no register
+// BM x BN tile at a time and walks its share of the list:
+//   * buffer_load_dwordx4 ... lds streams the operand tiles straight into an LDS ring (no register
 //     staging) in k-blocks of BK = 64, so every request is a full 128-byte line of one operand
 //     row; the ring keeps a block and a half in flight while the current one is multiplied;
 //   * LDS rows are 128 bytes (8 chunks of 16 bytes); chunk c of row r sits at position
 //     c ^ ((r >> 1) & 7), so the 1 KiB-contiguous DMA writes and the ds_read_b128 fragment reads
-//     are both bank-conflict free;
+//     are both bank-conflict free (a k-major operand: rows of 2 BN bytes, 64-byte blocks
+//     XOR-swizzled with row & 3, read with ds_read_b64_tr_b16);
 //   * each wave owns a 128 x 64 (or 64 x 64) sub-tile as 32 x 32 v_mfma_f32_32x32x16_bf16 tiles
 //     with fp32 accumulation;
 //   * the epilogue moves tiles between the "lane owns a column" accumulator layout and the
 //     "lane owns a row" layout with two MFMAs against a permuted identity, so that the addend is
-//     read and both output orientations are written with wide, coalesced accesses staged through
-//     wave-private LDS.
+//     read and the outputs are written with wide, coalesced accesses staged through wave-private
+//     LDS.
 #include <stdlib.h>
 
 #include "common.h"
