@@ -20,18 +20,23 @@ _ENGINE_CACHE_MAX = 4     # each cached engine holds its bf16 workspace
 _CACHE_LOCK = threading.Lock()
 
 
-def _cached(key, make):
+_PRODUCT_CACHE: "OrderedDict[tuple, object]" = OrderedDict()      # job tables of the stand-alone products: small
+_PRODUCT_CACHE_MAX = 64
+
+
+def _cached(key, make, cache=None, limit=_ENGINE_CACHE_MAX):
+    cache = _ENGINE_CACHE if cache is None else cache
     with _CACHE_LOCK:
-        eng = _ENGINE_CACHE.get(key)
+        eng = cache.get(key)
         if eng is None:
             eng = make()
             eng._fn_lock = threading.Lock()       # one caller at a time enqueues on this engine
             eng._fn_done = None                   # event after the launches of its last call
-            _ENGINE_CACHE[key] = eng
-            while len(_ENGINE_CACHE) > _ENGINE_CACHE_MAX:
-                _ENGINE_CACHE.popitem(last=False)
+            cache[key] = eng
+            while len(cache) > limit:
+                cache.popitem(last=False)
         else:
-            _ENGINE_CACHE.move_to_end(key)
+            cache.move_to_end(key)
         return eng
 
 
@@ -58,6 +63,7 @@ def clear_engine_cache() -> None:
     """Drop the workspaces cached by the functional entry points."""
     with _CACHE_LOCK:
         _ENGINE_CACHE.clear()
+        _PRODUCT_CACHE.clear()
 
 
 def _rounding_flag(rounding: str) -> bool:

@@ -14,6 +14,8 @@ implementation (all citations are into /root/reference/muon.py):
                              built on the Triton kernels muon.py:349-746; see its docstring
                              for what of it can and cannot be pinned)
   ns_aol4_rows               the same with muon.py:785 (`A / s`, rows only) taken as written
+  ns_line_1 / _2 / _3        muon.py:420-457, 547-588, 705-745  (the three products as operators of
+                             their own: A A^T, alpha A A^T + beta A, a X + B X)
   muon_update                muon.py:8-15
   adam_update                muon.py:104-109
   OracleSingleDeviceMuon     muon.py:73-101
@@ -52,6 +54,15 @@ What pins each function (the reference ships no tests, golden vectors or fixture
                      diagonal case.  PARITY UNPINNED against the reference's live code for the
                      same reasons as ns_aol4; in addition the reference's mirrored store makes
                      its own output depend on the autotuned block size, which is not restated.
+  * ns_line_1/2/3 -- what each computes is pinned by float64 matrix products and by the special
+                     cases that single out each term and each scalar (alpha = 0, beta = 0, a = 0,
+                     B = 0, B = I, a row-scaled A whose two triangles differ); ns_aol4, built from
+                     them, is pinned as above.  Their rounding against the reference's live
+                     kernels (which run only under Triton on a GPU) is PARITY UNPINNED: fp32
+                     accumulation and one cast at the store are what the kernels' source states
+                     (muon.py:388-400, 512-536, 694-696); the order of the fp32 sums and, for
+                     ns_line_3, the type in which the kernel forms `X * alpha` (muon.py:679-685) are
+                     the compiler's.
 No other function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -93,6 +104,36 @@ def _upper_mirrored(F: torch.Tensor) -> torch.Tensor:
     return torch.triu(F) + torch.triu(F, 1).mT
 
 
+def _acc_dtype(t: torch.Tensor) -> torch.dtype:
+    return torch.float64 if t.dtype == torch.float64 else torch.float32
+
+
+def ns_line_1(A: torch.Tensor) -> torch.Tensor:
+    """C = A @ A.T, muon.py:420-457: the kernel accumulates in fp32 and casts once to the tensor's
+    dtype (muon.py:388-400), and stores every block on or above the diagonal together with its
+    mirror image (muon.py:374-378, 402-413).  A is (M, K) or (batch, M, K)."""
+    acc = _acc_dtype(A)
+    return _upper_mirrored((A.to(acc) @ A.to(acc).mT).to(A.dtype))
+
+
+def ns_line_2(A: torch.Tensor, alpha: float, beta: float) -> torch.Tensor:
+    """C = alpha * A @ A.T + beta * A for a symmetric square A, muon.py:547-588: fp32 accumulation of
+    the product, alpha and beta applied in fp32, one cast (muon.py:512-536), mirrored store
+    (muon.py:538-552)."""
+    acc = _acc_dtype(A)
+    Af = A.to(acc)
+    return _upper_mirrored((alpha * (Af @ Af.mT) + beta * Af).to(A.dtype))
+
+
+def ns_line_3(B: torch.Tensor, X: torch.Tensor, a: float) -> torch.Tensor:
+    """C = a * X + B @ X, muon.py:705-745, by the formula of its docstring (muon.py:707) in fp32 with
+    one cast at the store (muon.py:694-696).  (The kernel seeds its accumulator with `X * alpha`
+    evaluated by Triton's scalar promotion before the fp32 cast, muon.py:679-685: in which type that
+    product is taken is the compiler's rule, not restated; PARITY UNPINNED against the live kernel.)"""
+    acc = _acc_dtype(X)
+    return (a * X.to(acc) + B.to(acc) @ X.to(acc)).to(X.dtype)
+
+
 def ns_aol4(G: torch.Tensor, epsilon: float = 1e-7, work_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """The 4-iteration AOL-rescaled variant, muon.py:748-799, with the Gram matrix rescaled on
     both sides (see the module docstring).  Every Triton kernel of the reference accumulates in
@@ -105,18 +146,16 @@ def ns_aol4(G: torch.Tensor, epsilon: float = 1e-7, work_dtype: torch.dtype = to
     tall = G.size(-2) > G.size(-1)
     if tall:                                                       # muon.py:761-762
         X = X.mT
-    gram = lambda Y: _upper_mirrored((Y.to(acc) @ Y.to(acc).mT).to(work_dtype))      # ns_line_1
-    A = gram(X)                                                    # muon.py:778
+    A = ns_line_1(X)                                               # muon.py:778
     s = torch.clamp_min(A.to(acc).abs().sum(dim=-1, keepdim=True).to(work_dtype).to(acc), epsilon)  # muon.py:779-781
     r = torch.rsqrt(s)
     X = (X.to(acc) * r).to(work_dtype)                             # muon.py:782
     A = (A.to(acc) * (r * r.mT)).to(work_dtype)                    # muon.py:785, on both sides
     for it, (a, b, c) in enumerate(AOL_CONSTS):
         if it > 0:
-            A = gram(X)                                            # muon.py:792
-        Af = A.to(acc)
-        B = _upper_mirrored((c * (Af @ Af.mT) + b * Af).to(work_dtype))               # ns_line_2, muon.py:786, 793
-        X = (a * X.to(acc) + B.to(acc) @ X.to(acc)).to(work_dtype)                    # ns_line_3, muon.py:787, 794
+            A = ns_line_1(X)                                       # muon.py:792
+        B = ns_line_2(A, alpha=c, beta=b)                          # muon.py:786, 793
+        X = ns_line_3(B, X, a)                                     # muon.py:787, 794
     if tall:                                                       # muon.py:797-798
         X = X.mT
     return X

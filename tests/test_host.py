@@ -341,6 +341,54 @@ def test_reference_module_name_is_importable():
     z = inspect.signature(muon.zeropower_via_newtonschulz5).parameters
     assert z["steps"].default == 5 and z["epsilon"].default == 1e-7
     assert plan.NS_COEFFS == (3.4445, -4.7750, 2.0315)
+    # the three products as operators: muon.py:420, 547, 705
+    K = inspect.Parameter.KEYWORD_ONLY
+    for fn, names in ((muon.ns_line_1, ["A", "out"]), (muon.ns_line_2, ["A", "alpha", "beta", "out"]),
+                      (muon.ns_line_3, ["B", "X", "a", "out"])):
+        ps = inspect.signature(fn).parameters
+        assert list(ps) == names and ps["out"].kind == K and ps["out"].default is None
+        assert all(ps[n].default is inspect.Parameter.empty for n in names[:-1])
+
+
+def test_product_operators_check_shapes_before_anything_else_and_their_job_lists_validate():
+    import muon
+    from muon_amd import ops
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="must be 2D or 3D, but got 4D"):        # muon.py:424-425
+        muon.ns_line_1(z(2, 2, 4, 4))
+    with pytest.raises(ValueError, match="symmetric square matrix"):             # muon.py:555-558
+        muon.ns_line_2(z(4, 6), 1.0, 1.0)
+    with pytest.raises(ValueError, match="B must be square"):                    # muon.py:710-711
+        muon.ns_line_3(z(4, 6), z(4, 6), 1.0)
+    with pytest.raises(ValueError, match="same number of rows"):                 # muon.py:713-714
+        muon.ns_line_3(z(4, 4), z(6, 6), 1.0)
+    with pytest.raises(muon_amd.MuonAmdError, match="no CPU implementation"):
+        muon.ns_line_1(z(4, 4))
+    # the job list of a product: every tile on or above the diagonal once (mirrored products) or every
+    # tile once, each over the whole reduction, in an order the library accepts
+    lib = _lib.load()
+    for tile_class, batch, rows_p, cols_p, kdim, sym in ((0, 3, 384, 384, 192, True), (1, 2, 1024, 1024, 1024, True),
+                                                         (0, 1, 256, 640, 256, False), (1, 2, 1280, 1536, 1280, False)):
+        jobs = ops._product_jobs(tile_class, batch, rows_p, cols_p, kdim, sym)
+        T = plan.TILE_DIMS[tile_class][0]
+        mt, nt = rows_p // T, cols_p // T
+        assert len(jobs) == batch * (mt * (mt + 1) // 2 if sym else mt * nt)
+        assert len({(j["desc"], j["i0"], j["j0"]) for j in jobs}) == len(jobs)
+        assert (jobs["k0"] == 0).all() and (jobs["k1"] == kdim).all() and (jobs["split"] == 0).all()
+        if sym:
+            assert (jobs["j0"] >= jobs["i0"]).all() and ((jobs["i0"] == jobs["j0"]) == (jobs["diag"] == 1)).all()
+        d = np.zeros(batch, dtype=_lib.GEMM_DESC)
+        d["P"] = d["Q"] = 1 << 20
+        d["C"] = 1 << 24
+        if sym:
+            d["CT"] = d["C"]
+        d["ldp"] = kdim
+        d["ldq"] = kdim if sym else cols_p
+        d["q_kmajor"] = 0 if sym else 1
+        d["ldc"] = d["ldct"] = cols_p
+        d["K"], d["rows"], d["colsn"] = kdim, rows_p, cols_p
+        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(d), batch, _lib.host_ptr(jobs), len(jobs), tile_class, 0)
+        assert rc == 0, lib.muon_amd_last_error()
 
 
 def test_product_never_imports_the_oracle():

@@ -353,3 +353,65 @@ def test_aol4_golden_fixture_is_what_the_oracle_computes(golden_dir):
         want = torch.from_numpy(z[name + "/bf16"].astype(np.int16)).view(torch.bfloat16)
         assert O.rel_fro(got.float(), want.float()) < 1e-6, name        # bf16 CPU matmuls are deterministic here
         assert O.rel_fro(got.double(), z[name + "/fp64_closed_form"]) < 2e-2, name
+
+
+# ------------------------------------------------------------------------------------------
+# the three products as operators of their own (muon.py:420-457, 547-588, 705-745)
+# ------------------------------------------------------------------------------------------
+def test_product_operators_against_brute_force_and_the_cases_that_single_out_each_term():
+    g = torch.Generator().manual_seed(21)
+    A = torch.randn(5, 7, dtype=torch.float64, generator=g)
+    S = torch.randn(6, 6, dtype=torch.float64, generator=g)
+    S = S + S.mT
+    X = torch.randn(6, 4, dtype=torch.float64, generator=g)
+    T = lambda M: [list(col) for col in zip(*M)]
+    mm = lambda P, Q: torch.tensor(O.matmul_brute_force(P.tolist(), Q.tolist()), dtype=torch.float64)
+    # float64 in, float64 arithmetic: the formulas themselves (a transposed operand, a swapped pair of
+    # scalars or a dropped term fails one of these)
+    assert (O.ns_line_1(A) - mm(A, A.mT)).abs().max() < 1e-12                     # 5 x 5, not A^T A (7 x 7)
+    assert O.ns_line_1(A).shape == (5, 5)
+    assert (O.ns_line_2(S, 2.0, -3.0) - (2.0 * mm(S, S) - 3.0 * S)).abs().max() < 1e-12
+    assert (O.ns_line_2(S, 0.0, 1.5) - 1.5 * S).abs().max() < 1e-12               # beta goes with A
+    assert (O.ns_line_2(S, 1.0, 0.0) - O.ns_line_1(S)).abs().max() < 1e-12        # alpha with the product
+    assert (O.ns_line_3(S, X, 0.5) - (0.5 * X + mm(S, X))).abs().max() < 1e-12    # B X, not X B or B^T... (S symmetric)
+    R = torch.randn(6, 6, dtype=torch.float64, generator=g)                       # a non-symmetric B tells B X from B^T X
+    assert (O.ns_line_3(R, X, 0.0) - mm(R, X)).abs().max() < 1e-12
+    assert (O.ns_line_3(torch.zeros(6, 6, dtype=torch.float64), X, -2.0) + 2.0 * X).abs().max() < 1e-12
+    assert (O.ns_line_3(torch.eye(6, dtype=torch.float64), X, 3.0) - 4.0 * X).abs().max() < 1e-12
+    # the mirrored store (muon.py:402-413, 538-552): what is below the diagonal is the image of what
+    # is above it, also for an input whose two triangles differ
+    N = S * torch.tensor([1.0, 1.2, 0.8, 1.1, 0.9, 1.0], dtype=torch.float64)[:, None]
+    got = O.ns_line_2(N, 1.0, 1.0)
+    full = mm(N, N.mT) + N
+    assert (torch.triu(got) - torch.triu(full)).abs().max() < 1e-12
+    assert (got - got.mT).abs().max() == 0 and (full - full.mT).abs().max() > 1e-2
+    # a batch is its matrices one by one
+    Ab = torch.randn(3, 4, 9, dtype=torch.float64, generator=g)
+    for k in range(3):
+        assert (O.ns_line_1(Ab)[k] - O.ns_line_1(Ab[k])).abs().max() < 1e-12
+    # bf16 storage: fp32 accumulation and one rounding -> within half a bf16 step of the exact value
+    Ah = torch.randn(40, 72, generator=g).bfloat16()
+    exact = Ah.double() @ Ah.double().mT
+    got = O.ns_line_1(Ah)
+    assert got.dtype == torch.bfloat16
+    assert ((got.double() - exact).abs() <= 2.0 ** -8 * exact.abs() * 1.001 + 1e-5).all()
+    Sh = O.ns_line_1((torch.randn(48, 48, generator=g) / 7).bfloat16())            # symmetric bf16 input
+    exact = -4.775 * Sh.double() + 2.0315 * Sh.double() @ Sh.double()
+    got = O.ns_line_2(Sh, 2.0315, -4.775)
+    assert ((got.double() - exact).abs() <= 2.0 ** -8 * exact.abs() * 1.001 + 1e-4).all()
+    Xh = torch.randn(48, 80, generator=g).bfloat16()
+    exact = 3.4445 * Xh.double() + Sh.double() @ Xh.double()
+    got = O.ns_line_3(Sh, Xh, 3.4445)
+    assert ((got.double() - exact).abs() <= 2.0 ** -8 * exact.abs() * 1.001 + 1e-4).all()
+
+
+def test_newton_schulz_iteration_built_from_the_product_operators():
+    """muon.py:285-287 written with the three operators (as muon.py:789-794 does) is the iteration
+    of the specification: in float64 the two agree to rounding."""
+    G = torch.randn(12, 20, dtype=torch.float64, generator=torch.Generator().manual_seed(22))
+    X = G / (G.norm() + 1e-7)
+    for _ in range(5):
+        A = O.ns_line_1(X)
+        B = O.ns_line_2(A, alpha=C_, beta=B_)
+        X = O.ns_line_3(B, X, A_)
+    assert (X - O._ns5(G, 5, 1e-7, torch.float64)).abs().max() < 1e-12
