@@ -110,7 +110,13 @@ def zeropower_via_newtonschulz5(G: torch.Tensor, steps: int = 5, epsilon: float 
 
     rounding="reference" rounds to bf16 wherever the reference's bf16 tensor expression does;
     "fused" rounds once per stored matrix (closer to the fp32 result).
+
+    The second positional argument is the iteration count, as in the specification
+    (muon.py:265-266); the reference's live function takes epsilon there (muon.py:749), so a
+    non-integral value in that place is refused rather than truncated to zero iterations.
     """
+    if isinstance(steps, bool) or int(steps) != steps or steps < 0:
+        raise TypeError(f"steps must be a non-negative integer, got {steps!r} (pass epsilon by keyword)")
     return _orthogonalise(G, steps, epsilon, _rounding_flag(rounding), "ns5")
 
 

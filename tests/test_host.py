@@ -326,6 +326,11 @@ def test_no_cpu_fallback():
         muon_amd.muon_update(torch.ones(4, 8), torch.zeros(4, 8))
     with pytest.raises(AssertionError):
         muon_amd.zeropower_via_newtonschulz5(torch.ones(4))                                  # muon.py:275
+    # the live function's second positional argument is epsilon (muon.py:749), the specification's the
+    # iteration count (muon.py:265): an epsilon in that place must not become zero iterations
+    for bad in (1e-7, 2.5, -1):
+        with pytest.raises(TypeError, match="steps must be a non-negative integer"):
+            muon_amd.zeropower_via_newtonschulz5(torch.ones(4, 8), bad)
 
 
 def test_reference_module_name_is_importable():
