@@ -191,6 +191,11 @@ def ns_line_3(B: torch.Tensor, X: torch.Tensor, a: float, *, out: torch.Tensor =
     tile_class = _plan.tile_class_for(min(M, N))
     unit = _plan.pad_unit(tile_class)
     mp, np_ = _plan._round_up(M, unit), _plan._round_up(N, unit)
+    # as in the optimizer's update launches: 256 x 256 tiles also for shorter matrices when their
+    # padded sizes allow it and there are enough of them to give every CU one
+    if (tile_class == 0 and mp % 256 == 0 and np_ % 256 == 0 and
+            batch * (mp // 256) * (np_ // 256) >= _plan.RESIDENT_BIG_TILE_WORKGROUPS):
+        tile_class = 1
     with torch.cuda.device(X.device):
         prod = _cached(("update_product", X.device, tile_class, batch, mp, np_),
                        lambda: _Product(X.device, tile_class, batch, mp, np_, mp, False),
