@@ -439,6 +439,57 @@ def secondary(name, gates):
     return out
 
 
+def product_operators(gates):
+    """The three products as operators of their own (ns_line_1 / ns_line_2 / ns_line_3, reference
+    muon.py:420, 547, 705) on the shapes of the Llama-3-8B feed-forward matrices: checked against
+    the oracle on a small ragged case first, then timed with HIP events (results written into
+    buffers given by the caller, as the reference's iteration does, muon.py:789-794)."""
+    import muon_amd
+    from oracle import muon_oracle as O
+
+    out = {}
+    dev = torch.device("cuda:0")
+    if gates:
+        g = torch.Generator().manual_seed(99)
+        X = (torch.randn(2, 200, 328, generator=g) * 0.05).bfloat16()
+        S = O.ns_line_1(X)
+        worst = 0.0
+        for name, got, want in (
+                ("ns_line_1", muon_amd.ns_line_1(X.to(dev)), S),
+                ("ns_line_2", muon_amd.ns_line_2(S.to(dev), 2.0315, -4.7750), O.ns_line_2(S, 2.0315, -4.7750)),
+                ("ns_line_3", muon_amd.ns_line_3(S.to(dev), X.to(dev), 3.4445), O.ns_line_3(S, X, 3.4445))):
+            d = (got.double().cpu() - want.double()).abs()
+            step = 2.0 ** -7 * want.double().abs() + 1e-4            # one bf16 step at the value
+            if not (d <= step).all():
+                sys.exit(f"bench.py: correctness gate failed before timing: {name} is more than one bf16 step from the oracle")
+            worst = max(worst, float((d / step).max()))
+        out["gate_max_bf16_steps_from_oracle"] = round(worst, 3)
+    b, m, n = 16, 4096, 14336
+    X = (torch.randn(b, m, n, device=dev) * 0.01).bfloat16()
+    A = torch.empty(b, m, m, device=dev, dtype=torch.bfloat16)
+    B = torch.empty_like(A)
+    C = torch.empty_like(X)
+    calls = (("ns_line_1", lambda: muon_amd.ns_line_1(X, out=A), b * m * (m + 1) * n),
+             ("ns_line_2", lambda: muon_amd.ns_line_2(A, 2.0315, -4.7750, out=B), b * m * m * (m + 1)),
+             ("ns_line_3", lambda: muon_amd.ns_line_3(B, X, 3.4445, out=C), 2 * b * m * m * n))
+    out["shape"] = f"{b} x ({m} x {n}), bf16; flops: the minimum given symmetry"
+    for name, call, flops in calls:
+        call()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 3
+        out[name] = {"ms": round(ms, 3), "tflops": round(flops / ms / 1e9, 1),
+                     "frac_of_peak": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    del X, A, B, C
+    muon_amd.clear_engine_cache()
+    torch.cuda.empty_cache()
+    return out
+
+
 # ------------------------------------------------------------------------------------------
 # Library baseline on the same GPU: the reference's step written with torch operations (bf16
 # torch.matmul = rocBLAS / hipBLASLt for the Newton-Schulz products, one parameter after the other,
@@ -692,6 +743,7 @@ def main():
         line["gpt2_124m"] = secondary("gpt2-124m", not args.no_gates)
         line["ns32"] = secondary("ns32", not args.no_gates)
         line["conv"] = secondary("conv", not args.no_gates)
+        line["product_operators"] = product_operators(not args.no_gates)
     if not args.no_torch_baseline:
         line["torch_gpu_baseline"] = torch_gpu_baseline(args.workload)
         line["torch_gpu_baseline"]["speedup"] = round(line["torch_gpu_baseline"]["ms_per_step"] / res["ms_per_step"], 2)
