@@ -28,26 +28,41 @@ from .engine import _Staging, _stream_ptr, _upload, require_gpu_tensor
 from .functional import _PRODUCT_CACHE, _PRODUCT_CACHE_MAX, _cached, _exclusive
 
 
-def _product_jobs(tile_class: int, batch: int, rows_p: int, cols_p: int, kdim: int, sym: bool) -> np.ndarray:
+def _product_jobs(tile_class: int, batch: int, rows_p: int, cols_p: int, kdim: int, sym: bool,
+                  nsplit: int = 1) -> np.ndarray:
     """One job per output tile and matrix (for a mirrored product: per tile on or above the
-    diagonal), each over the whole reduction, in super-block order dealt to the XCDs."""
+    diagonal), in super-block order dealt to the XCDs.  nsplit > 1: the reduction of every tile is
+    shared by nsplit jobs that meet in a group of fp32 slots (tile t of the launch: slots
+    t * nsplit ..), as the optimizer does for the X X^T of short, very wide matrices."""
     TR, TC = _plan.TILE_DIMS[tile_class]
     si, sj = _plan.SUPER_DIMS[tile_class]
     ti, tj = _plan._tile_order(rows_p // TR, cols_p // TC, sym, TR // TC, si, sj)
-    one = np.zeros(len(ti), dtype=_lib.TILE_JOB)
-    one["i0"], one["j0"], one["k1"] = ti * TR, tj * TC, kdim
+    one = np.zeros(len(ti) * nsplit, dtype=_lib.TILE_JOB)
+    one["i0"], one["j0"] = np.repeat(ti * TR, nsplit), np.repeat(tj * TC, nsplit)
     if sym:
-        one["diag"] = (ti == tj // (TR // TC)).astype(np.int32)
+        one["diag"] = np.repeat((ti == tj // (TR // TC)).astype(np.int32), nsplit)
+    if nsplit == 1:
+        one["k1"] = kdim
+    else:
+        edges = (np.arange(nsplit + 1) * (kdim // _plan.GEMM_BK) // nsplit) * _plan.GEMM_BK
+        idx = np.tile(np.arange(nsplit), len(ti))
+        one["k0"], one["k1"] = edges[idx], edges[idx + 1]
+        one["part_base"] = np.repeat(np.arange(len(ti)) * nsplit, nsplit)
+        one["split"] = idx | (nsplit << 16)
     jobs = np.tile(one, batch)
     jobs["desc"] = np.repeat(np.arange(batch, dtype=np.int32), len(one))
+    if nsplit > 1:
+        jobs["part_base"] += np.repeat(np.arange(batch) * len(ti) * nsplit, len(one))
     return np.ascontiguousarray(jobs[_plan.xcd_permutation(len(jobs), si * sj)])
 
 
 class _Product:
-    """Job list (uploaded once) and descriptor buffer of one product shape on one device."""
+    """Job list (uploaded once), descriptor buffer and, for split reductions, the fp32 slots and
+    their counters, of one product shape on one device."""
 
-    def __init__(self, device, tile_class: int, batch: int, rows_p: int, cols_p: int, kdim: int, sym: bool):
-        self.jobs = _product_jobs(tile_class, batch, rows_p, cols_p, kdim, sym)
+    def __init__(self, device, tile_class: int, batch: int, rows_p: int, cols_p: int, kdim: int, sym: bool,
+                 nsplit: int = 1):
+        self.jobs = _product_jobs(tile_class, batch, rows_p, cols_p, kdim, sym, nsplit)
         self.device = device
         self.tile_class = tile_class
         self.batch = batch
@@ -55,17 +70,26 @@ class _Product:
         self.desc_dev = torch.empty(batch * _lib.GEMM_DESC.itemsize, dtype=torch.uint8, device=device)
         self.staging = _Staging(device)
         self.desc_key = None
+        self.split_slots = len(self.jobs) if nsplit > 1 else 0
+        if self.split_slots:
+            TR, TC = _plan.TILE_DIMS[tile_class]
+            self.partials = torch.empty(self.split_slots * TR * TC, dtype=torch.float32, device=device)
+            self.counters = torch.zeros(self.split_slots, dtype=torch.int32, device=device)
 
     def launch(self, descs: np.ndarray, alpha: float, beta: float, flags: int) -> None:
         lib = _lib.load()
         key = descs.tobytes()
         if key != self.desc_key:          # the same tensors as last time (a loop over fixed buffers): nothing to redo
             _lib.check(lib.muon_amd_validate_gemm(_lib.host_ptr(descs), self.batch, _lib.host_ptr(self.jobs),
-                                                  len(self.jobs), self.tile_class, 0), "validate_gemm")
+                                                  len(self.jobs), self.tile_class, self.split_slots), "validate_gemm")
             self.staging.upload(descs, self.desc_dev)
             self.desc_key = key
+        partials = counters = None
+        if self.split_slots:
+            self.counters.zero_()         # every launch leaves them zero; a launch that died must not poison the next
+            partials, counters = self.partials.data_ptr(), self.counters.data_ptr()
         _lib.check(lib.muon_amd_ns_gemm(self.desc_dev.data_ptr(), self.jobs_dev.data_ptr(), len(self.jobs),
-                                        self.tile_class, alpha, beta, 0.0, flags, None, None,
+                                        self.tile_class, alpha, beta, 0.0, flags, partials, counters,
                                         _stream_ptr(self.device)), "ns_gemm")
 
 
@@ -128,8 +152,10 @@ def _symmetric_product(A: torch.Tensor, out, alpha: float, beta: float, addend: 
     mp = _plan._round_up(M, unit)
     kp = mp if addend else _plan._round_up(K, _plan.GEMM_BK)
     with torch.cuda.device(A.device):
-        prod = _cached(("sym_product", A.device, tile_class, batch, mp, kp),
-                       lambda: _Product(A.device, tile_class, batch, mp, mp, kp, True),
+        # X X^T of a short, very wide matrix: a few tiles with very long reductions, which are split
+        nsplit = 1 if addend or tile_class != 0 else _plan.split_factor(mp, kp)
+        prod = _cached(("sym_product", A.device, tile_class, batch, mp, kp, nsplit),
+                       lambda: _Product(A.device, tile_class, batch, mp, mp, kp, True, nsplit),
                        _PRODUCT_CACHE, _PRODUCT_CACHE_MAX)
         with _exclusive(prod, A.device):
             src = _padded(A3, mp, kp)

@@ -49,7 +49,8 @@ def _sym(shape, seed):
     return ((R + R.mT) / 2).bfloat16()
 
 
-LINE1_SHAPES = [(128, 64), (100, 200), (5, 3), (768, 3072), (1024, 4096), (1300, 520), (3, 200, 136), (2, 1024, 1024)]
+LINE1_SHAPES = [(128, 64), (100, 200), (5, 3), (768, 3072), (1024, 4096), (1300, 520), (3, 200, 136), (2, 1024, 1024),
+                (128, 16384), (3, 200, 8200), (512, 4608)]      # short and very wide: split reductions
 
 
 @pytest.mark.parametrize("shape", LINE1_SHAPES)

@@ -372,14 +372,20 @@ def test_product_operators_check_shapes_before_anything_else_and_their_job_lists
     # the job list of a product: every tile on or above the diagonal once (mirrored products) or every
     # tile once, each over the whole reduction, in an order the library accepts
     lib = _lib.load()
-    for tile_class, batch, rows_p, cols_p, kdim, sym in ((0, 3, 384, 384, 192, True), (1, 2, 1024, 1024, 1024, True),
-                                                         (0, 1, 256, 640, 256, False), (1, 2, 1280, 1536, 1280, False)):
-        jobs = ops._product_jobs(tile_class, batch, rows_p, cols_p, kdim, sym)
+    for tile_class, batch, rows_p, cols_p, kdim, sym, nsplit in (
+            (0, 3, 384, 384, 192, True, 1), (1, 2, 1024, 1024, 1024, True, 1), (0, 1, 256, 640, 256, False, 1),
+            (1, 2, 1280, 1536, 1280, False, 1), (0, 1, 128, 128, 16384, True, 10), (0, 3, 256, 256, 8256, True, 5)):
+        jobs = ops._product_jobs(tile_class, batch, rows_p, cols_p, kdim, sym, nsplit)
         T = plan.TILE_DIMS[tile_class][0]
         mt, nt = rows_p // T, cols_p // T
-        assert len(jobs) == batch * (mt * (mt + 1) // 2 if sym else mt * nt)
-        assert len({(j["desc"], j["i0"], j["j0"]) for j in jobs}) == len(jobs)
-        assert (jobs["k0"] == 0).all() and (jobs["k1"] == kdim).all() and (jobs["split"] == 0).all()
+        assert len(jobs) == batch * (mt * (mt + 1) // 2 if sym else mt * nt) * nsplit
+        assert len({(j["desc"], j["i0"], j["j0"], j["k0"]) for j in jobs}) == len(jobs)
+        if nsplit == 1:
+            assert (jobs["k0"] == 0).all() and (jobs["k1"] == kdim).all() and (jobs["split"] == 0).all()
+        else:       # every job its own slot; the jobs of a tile cover its reduction once
+            assert sorted(jobs["part_base"] + (jobs["split"] & 0xffff)) == list(range(len(jobs)))
+            assert ((jobs["split"] >> 16) == nsplit).all()
+            assert int((jobs["k1"] - jobs["k0"]).sum()) == kdim * len(jobs) // nsplit
         if sym:
             assert (jobs["j0"] >= jobs["i0"]).all() and ((jobs["i0"] == jobs["j0"]) == (jobs["diag"] == 1)).all()
         d = np.zeros(batch, dtype=_lib.GEMM_DESC)
@@ -392,7 +398,8 @@ def test_product_operators_check_shapes_before_anything_else_and_their_job_lists
         d["q_kmajor"] = 0 if sym else 1
         d["ldc"] = d["ldct"] = cols_p
         d["K"], d["rows"], d["colsn"] = kdim, rows_p, cols_p
-        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(d), batch, _lib.host_ptr(jobs), len(jobs), tile_class, 0)
+        rc = lib.muon_amd_validate_gemm(_lib.host_ptr(d), batch, _lib.host_ptr(jobs), len(jobs), tile_class,
+                                        len(jobs) if nsplit > 1 else 0)
         assert rc == 0, lib.muon_amd_last_error()
 
 
