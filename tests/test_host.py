@@ -577,3 +577,28 @@ def test_rows_only_aol_is_refused_below_its_stated_size():
         assert plan.plan_chunks([(256, 256), shape], 4, False, 1 << 30, "aol4")
         assert plan.plan_chunks([(256, 256), shape], 5, True, 1 << 30, "ns5")
     assert plan.plan_chunks([(plan.AOL_ROWS_MIN_SIDE, 63)], 4, False, 1 << 30, "aol4_rows")
+
+
+def test_update_launches_of_matrices_with_ragged_super_blocks_deal_whole_matrices_to_the_xcds():
+    """Three tile rows (m = 768) against the super-block's four: the 256 x 256 update list is dealt
+    in groups of 108 jobs = 4, 12 or 3 whole matrices, so an XCD sees few matrices; matrices whose
+    tile rows fill the super-blocks (m = 1024, 4096) keep the super-block groups."""
+    assert plan.whole_matrix_group([27, 9, 36, 36], 32) == 108
+    assert plan.whole_matrix_group([75, 25, 100], 32) == 100           # lcm 300 is more than eight super-blocks
+    gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    (c,) = plan.plan_chunks(gpt2, 5, True, 16 << 30)
+    assert c.update_class == 1 and len(c.full_jobs) == 1296
+    x = np.arange(1296) % 8
+    per_xcd = [len(set(c.full_jobs["desc"][x == k].tolist())) for k in range(8)]
+    assert max(per_xcd) <= 9 and sum(per_xcd) == 48                     # no matrix on two XCDs
+    assert sorted(map(tuple, c.full_jobs[["desc", "i0", "j0"]].tolist())) == sorted(
+        (k, i, j) for k, lay in enumerate(c.layouts) for i in range(0, lay.mp, 256) for j in range(0, lay.np_, 256))
+    medium = [(1024, 3072), (1024, 1024), (1024, 4096), (4096, 1024)] * 4
+    (c,) = plan.plan_chunks(medium, 5, True, 16 << 30)
+    ref = c.full_jobs.copy()
+    old, plan.WHOLE_MATRIX_GROUPS = plan.WHOLE_MATRIX_GROUPS, False
+    try:
+        (c2,) = plan.plan_chunks(medium, 5, True, 16 << 30)
+    finally:
+        plan.WHOLE_MATRIX_GROUPS = old
+    assert (c2.full_jobs == ref).all()
