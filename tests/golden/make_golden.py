@@ -1,10 +1,11 @@
-"""Writes tests/golden/ns_golden.npz, step_golden.npz and aol4_golden.npz from the CPU oracle.
+"""Writes tests/golden/ns_golden.npz, step_golden.npz, aol4_golden.npz and ops_golden.npz from the CPU oracle.
 
 The reference ships no golden vectors and its Newton-Schulz contract (muon.py:265-291) is
 comment text, so these fixtures come from oracle/muon_oracle.py, whose functions are pinned by
 closed forms and invariants in tests/test_oracle.py.  Run from the repo root:
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py          # all of them
+    python tests/golden/make_golden.py ops      # ops_golden.npz alone
 """
 import os
 import sys
@@ -37,8 +38,35 @@ def aol4():
     np.savez_compressed(os.path.join(HERE, "aol4_golden.npz"), **out)
 
 
+def ops():
+    """Fixtures of the three product operators (oracle.ns_line_1/2/3, muon.py:420-457, 547-588, 705-745):
+    bf16 inputs, the oracle's bf16 results and the exact value of each expression (computed in
+    float64 from the bf16 operands the operator is given, stored as float32)."""
+    g = torch.Generator().manual_seed(20251127)
+    out = {}
+    for name, shape in [("small_24x40", (24, 40)), ("ragged_70x130", (70, 130)), ("batched_3x20x36", (3, 20, 36))]:
+        X = (torch.randn(*shape, generator=g) * 0.1).bfloat16()
+        A = O.ns_line_1(X)
+        B = O.ns_line_2(A, 2.0315, -4.7750)
+        C = O.ns_line_3(B, X, 3.4445)
+        Xd, Ad, Bd = X.double(), A.double(), B.double()
+        out[name + "/X"] = bf16_bits(X)
+        out[name + "/line1"] = bf16_bits(A)
+        out[name + "/line2"] = bf16_bits(B)
+        out[name + "/line3"] = bf16_bits(C)
+        out[name + "/line1_exact"] = (Xd @ Xd.mT).float().numpy()
+        out[name + "/line2_exact"] = (2.0315 * (Ad @ Ad.mT) - 4.7750 * Ad).float().numpy()
+        out[name + "/line3_exact"] = (3.4445 * Xd + Bd @ Xd).float().numpy()
+    np.savez_compressed(os.path.join(HERE, "ops_golden.npz"), **out)
+
+
 def main():
+    if sys.argv[1:] == ["ops"]:
+        ops()
+        print("wrote ops_golden.npz")
+        return
     aol4()
+    ops()
     torch.manual_seed(20251125)
     ns = {}
     for name, shape, std in [("wide_16x48", (16, 48), 1e-3), ("tall_48x16", (48, 16), 1e-3),

@@ -170,3 +170,21 @@ def test_newton_schulz_built_from_the_operators(M):
         else:
             for k in range(shape[0]):
                 assert O.rel_fro(X[k].float().cpu(), O.ns5_fp64_closed_form(G[k].double().numpy())) < 2e-2, (shape, k)
+
+
+def test_operators_against_the_golden_fixture(M, golden_dir):
+    """The committed vectors (tests/golden/ops_golden.npz, written by tests/golden/make_golden.py from
+    the oracle): each operator on the fixture's own bf16 inputs, within one bf16 step of the stored
+    result and within one rounding of the stored exact value."""
+    import os
+    import numpy as np
+    z = np.load(os.path.join(golden_dir, "ops_golden.npz"))
+    bf = lambda a: torch.from_numpy(a.astype(np.int16)).view(torch.bfloat16)
+    for name in sorted({k.split("/")[0] for k in z.files}):
+        X, A, B = bf(z[name + "/X"]), bf(z[name + "/line1"]), bf(z[name + "/line2"])
+        Xd, Ad, Bd = X.double().abs(), A.double().abs(), B.double().abs()
+        cases = (("line1", M.ns_line_1(X.cuda()), Xd @ Xd.mT),
+                 ("line2", M.ns_line_2(A.cuda(), 2.0315, -4.7750), 2.0315 * (Ad @ Ad.mT) + 4.7750 * Ad),
+                 ("line3", M.ns_line_3(B.cuda(), X.cuda(), 3.4445), 3.4445 * Xd + Bd @ Xd))
+        for key, got, terms in cases:
+            _check(got, torch.from_numpy(z[f"{name}/{key}_exact"]).double(), terms, bf(z[f"{name}/{key}"]), f"{name} {key}")

@@ -415,3 +415,24 @@ def test_newton_schulz_iteration_built_from_the_product_operators():
         B = O.ns_line_2(A, alpha=C_, beta=B_)
         X = O.ns_line_3(B, X, A_)
     assert (X - O._ns5(G, 5, 1e-7, torch.float64)).abs().max() < 1e-12
+
+
+def test_product_operator_golden_fixture_is_what_the_oracle_computes(golden_dir):
+    z = np.load(os.path.join(golden_dir, "ops_golden.npz"))
+    bf = lambda a: torch.from_numpy(a.astype(np.int16)).view(torch.bfloat16)
+    for name in sorted({k.split("/")[0] for k in z.files}):
+        X = bf(z[name + "/X"])
+        A = O.ns_line_1(X)
+        B = O.ns_line_2(A, 2.0315, -4.7750)
+        C = O.ns_line_3(B, X, 3.4445)
+        for got, key in ((A, "line1"), (B, "line2"), (C, "line3")):
+            want = bf(z[f"{name}/{key}"])
+            # the CPU's fp32 sums may come in another order on another host: at most one bf16 step, rarely
+            d = (got.double() - want.double()).abs()
+            assert (d <= 2.0 ** -7 * want.double().abs() + 1e-6).all(), (name, key)
+            assert (d != 0).double().mean() < 0.01, (name, key)
+            exact = torch.from_numpy(z[f"{name}/{key}_exact"]).double()
+            # one rounding of the exact value, plus what fp32 sums of these terms may be off by
+            Xd, Ad, Bd = X.double().abs(), bf(z[name + "/line1"]).double().abs(), bf(z[name + "/line2"]).double().abs()
+            terms = {"line1": Xd @ Xd.mT, "line2": 2.0315 * (Ad @ Ad.mT) + 4.7750 * Ad, "line3": 3.4445 * Xd + Bd @ Xd}[key]
+            assert ((want.double() - exact).abs() <= 2.0 ** -8 * 1.001 * exact.abs() + 2.0 ** -18 * terms).all(), (name, key)
