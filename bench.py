@@ -188,8 +188,23 @@ def correctness_gates(name):
 def run_optimizer_workload(name, steps, warmup, seed, ns_variant="ns5", use_graph=False, realloc_grads=False,
                            launch_events=True):
     import muon_amd
-    from muon_amd import engine
+    from muon_amd import engine, plan
 
+    # Per-launch events add up to the GEMM time only while launches run one after the other: the pass
+    # that records them keeps the matrices in one lane (a small model's matrices otherwise run as two
+    # lanes on two streams, whose launches overlap).
+    lanes_saved = plan.LANES
+    if launch_events and not use_graph:
+        plan.LANES = "1"
+    try:
+        return _run_optimizer_workload(muon_amd, engine, name, steps, warmup, seed, ns_variant, use_graph,
+                                       realloc_grads, launch_events)
+    finally:
+        plan.LANES = lanes_saved
+
+
+def _run_optimizer_workload(muon_amd, engine, name, steps, warmup, seed, ns_variant, use_graph, realloc_grads,
+                            launch_events):
     muon, adam, gstd, _, _ = workload_shapes(name)
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev)

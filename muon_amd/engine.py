@@ -1,6 +1,7 @@
 """Device-side driver of the grouped Muon / Adam launches (torch for memory and streams only)."""
 from __future__ import annotations
 
+import contextlib
 import os
 
 import numpy as np
@@ -308,18 +309,24 @@ class MuonGroupEngine:
     N_SCALARS = 4          # {1 - beta, beta, lr, 1 - lr * weight_decay}
 
     def __init__(self, shapes, device, steps: int = 5, reference_rounding: bool = True,
-                 workspace_cap: int | None = None, variant: str = "ns5"):
+                 workspace_cap: int | None = None, variant: str = "ns5", allow_lanes: bool = True):
         self.device = torch.device(device)
         with torch.cuda.device(self.device):
             _lib.check(_lib.load().muon_amd_init(), "init")
         self.shapes = [(int(r), int(c)) for r, c in shapes]
         cap = DEFAULT_WORKSPACE_CAP if workspace_cap is None else int(workspace_cap)
-        self.chunks = _plan.plan_chunks(self.shapes, steps, reference_rounding, cap, variant)
-        ws_bytes = max(c.workspace_bytes for c in self.chunks)
-        self.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=self.device)
-        base = self.workspace.data_ptr()
-        assert base % 256 == 0
-        self.runtimes = [_ChunkRuntime(c, base, self.device) for c in self.chunks]
+        # Lanes: disjoint sets of matrices with a workspace and (beyond the first, which runs on the
+        # caller's stream) a stream each; the chunks of a lane share its workspace and run back to back.
+        lanes = _plan.plan_lanes(self.shapes, steps, reference_rounding, cap, variant, allow_lanes)
+        self.chunks = [c for lane in lanes for c in lane]
+        self.workspaces = [torch.empty(max(c.workspace_bytes for c in lane), dtype=torch.uint8, device=self.device)
+                           for lane in lanes]
+        self.workspace = self.workspaces[0]
+        assert all(ws.data_ptr() % 256 == 0 for ws in self.workspaces)
+        self.lane_runtimes = [[_ChunkRuntime(c, ws.data_ptr(), self.device) for c in lane]
+                              for lane, ws in zip(lanes, self.workspaces)]
+        self.runtimes = [rt for lane in self.lane_runtimes for rt in lane]
+        self.lane_streams = [None] + [torch.cuda.Stream(self.device) for _ in lanes[1:]]      # default priority
         self._hyper = None
         # matrices whose momentum stage may run ahead of the step: those of the first chunk (the
         # later chunks reuse its workspace while the step runs); matrix index -> position in the chunk
@@ -365,10 +372,21 @@ class MuonGroupEngine:
         return (id(self), h["nesterov"], h["mutate_grad"], h["eps"], self._skip)
 
     def enqueue(self, scalars_ptr: int = 0):
+        """The launches of every lane: the first lane on the current stream, the others on their own
+        streams, which wait for what the current stream holds so far (the descriptor uploads of
+        `prepare`, the gradients) and which the current stream waits for before it goes on."""
         h = self._hyper
-        for n, rt in enumerate(self.runtimes):
-            rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
-                   h["wd_factor"], scalars_ptr=scalars_ptr, momentum_done=self._skip if n == 0 else frozenset())
+        main = torch.cuda.current_stream(self.device)
+        for side in self.lane_streams[1:]:
+            side.wait_stream(main)
+        for li, runtimes in enumerate(self.lane_runtimes):
+            with (torch.cuda.stream(self.lane_streams[li]) if li else contextlib.nullcontext()):
+                for n, rt in enumerate(runtimes):
+                    rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
+                           h["wd_factor"], scalars_ptr=scalars_ptr,
+                           momentum_done=self._skip if (li == 0 and n == 0) else frozenset())
+        for side in self.lane_streams[1:]:
+            main.wait_stream(side)
 
     def early_stream(self):
         """The side stream the early stages run on (default priority; created on first use)."""

@@ -247,8 +247,9 @@ class _MuonBase(torch.optim.Optimizer):
         if eng is None:
             self._muon_engines = {k: v for k, v in self._muon_engines.items() if k[0] != gi}
             with torch.cuda.device(device):
+                # (the stages that run during backward write into the first chunk's workspace: one lane)
                 eng = MuonGroupEngine(shapes, device, NS_STEPS, self._reference_rounding, self._workspace_bytes,
-                                      variant=self._ns_variant)
+                                      variant=self._ns_variant, allow_lanes=not self._overlap_backward)
             self._muon_engines[key] = eng
             self._graphs.pop(device, None)        # a recorded step refers to the engine that was replaced
         if self._overlap_backward:

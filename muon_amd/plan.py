@@ -484,11 +484,54 @@ class ChunkPlan:
         return 1.0, a, 0.0
 
 
-def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5"):
+def _shape_order_key(shapes, i):
+    return (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]), -shapes[i][0], i)
+
+
+LANES = os.environ.get("MUON_AMD_LANES", "auto")        # "auto", or a number of lanes to force ("1" switches them off)
+LANE_MIN_MATRICES = 8
+LANE_LAUNCH_US = (60.0, 1000.0)
+
+
+def plan_lanes(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5",
+               allow_lanes: bool = True):
+    """-> lanes, each a list of chunks.  Lanes have workspaces of their own and run side by side on
+    streams of their own, so that the launches of one fill the CUs that the last, partly filled
+    rounds of the other's leave idle (every launch is persistent: while one runs in full, the other
+    lane's next launch waits for CUs and starts where they free up).  Two lanes, each with every
+    other matrix of the sorted list, when the matrices make one chunk of at least 8 whose launches
+    are estimated at 60 us to 1 ms each: measured on the Muon part of a step, GPT-2-124M 2.07 ->
+    1.975 ms, 96 matrices of m = 512 1.60 -> 1.52, 96 of m = 1024 7.68 -> 7.51, 48 of m = 1280 7.10 ->
+    6.87 ms.  Not for short launches (the conv configuration: 0.43 -> 0.45 ms, and the host then
+    issues two streams' worth of them) nor for long ones (the Llama-3-8B matrices: 438 -> 448 ms; three
+    and four lanes were no better than two anywhere).  Which lane computes a matrix does not change
+    its bits."""
+    chunks = plan_chunks(shapes, steps, reference_rounding, workspace_cap, variant)
+    n = 1
+    if allow_lanes and LANES != "auto":
+        n = max(1, min(int(LANES), len(shapes)))
+    elif allow_lanes and len(chunks) == 1 and chunks[0].nmat >= LANE_MIN_MATRICES:
+        c = chunks[0]
+        est, _ = _chunk_time_us([(lay.rows, lay.cols) for lay in c.layouts], c.tile_class)
+        if LANE_LAUNCH_US[0] <= est / 3 <= LANE_LAUNCH_US[1]:
+            n = 2
+    if n == 1:
+        return [chunks]
+    order = sorted(range(len(shapes)), key=lambda i: _shape_order_key(shapes, i))
+    lanes = [plan_chunks(shapes, steps, reference_rounding, workspace_cap, variant, subset=order[k::n])
+             for k in range(n)]
+    if LANES == "auto" and any(c.update_class != chunks[0].update_class for lane in lanes for c in lane):
+        return [chunks]            # half the matrices would no longer fill the larger update tiles
+    return lanes
+
+
+def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5",
+                subset=None):
     """Split matrices [(rows, cols), ...] into chunks of one tile class each whose workspace (the bf16
     buffers and the scratch beside them) stays under `workspace_cap` bytes (a single matrix larger
     than the cap gets a chunk of its own).
-    Same-shape matrices are kept together so that their tiles batch into full waves of the GPU."""
+    Same-shape matrices are kept together so that their tiles batch into full waves of the GPU.
+    `subset`: positions in `shapes` to plan for (all of them when None)."""
     if variant == "aol4_rows":
         short = [tuple(sh) for sh in shapes if min(sh) < AOL_ROWS_MIN_SIDE]
         if short:
@@ -496,9 +539,7 @@ def plan_chunks(shapes, steps: int, reference_rounding: bool, workspace_cap: int
                 f"the rows-only AOL rescaling is not offered for matrices with a side below {AOL_ROWS_MIN_SIDE} "
                 f"(got {short[0][0]} x {short[0][1]}): the iteration does not contract there and amplifies rounding "
                 "differences without bound; use the symmetric rescaling (ns_variant='aol4', rescale='symmetric')")
-    order = sorted(range(len(shapes)),
-                   key=lambda i: (-tile_class_for(min(shapes[i])), -min(shapes[i]), -max(shapes[i]),
-                                  -shapes[i][0], i))
+    order = sorted(range(len(shapes)) if subset is None else subset, key=lambda i: _shape_order_key(shapes, i))
     need = [matrix_workspace_bytes(*shapes[i], pad_unit(tile_class_for(min(shapes[i])))) +
             matrix_scratch_bytes(*shapes[i], tile_class_for(min(shapes[i])), variant in ("aol4", "aol4_rows"))
             for i in order]

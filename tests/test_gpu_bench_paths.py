@@ -232,7 +232,7 @@ def test_large_tile_update_products_give_the_same_bits(M, monkeypatch):
             opt.step()
         torch.cuda.synchronize()
         (eng,) = opt._muon_engines.values()
-        assert [c.update_class for c in eng.chunks] == ([1] if mode == "auto" else [0])
+        assert {c.update_class for c in eng.chunks} == ({1} if mode == "auto" else {0})
         results[mode] = [p.detach().clone() for p in params]
     for a, b, s in zip(results["auto"], results["0"], shapes):
         assert torch.equal(a, b), s
@@ -274,3 +274,55 @@ def test_a_hundred_steps_stay_deterministic(M):
     for other in finals[1:]:
         for a, b in zip(finals[0], other):
             assert torch.equal(a, b)
+
+
+def test_two_lanes_give_the_bits_of_one_lane_eagerly_and_replayed(M):
+    """A parameter list run as two lanes (every other matrix of the sorted list, each lane with its own
+    workspace, the second on a stream of its own) ends bit for bit where the same list ends in one lane:
+    eagerly, replayed from a HIP graph (the second lane forks from and rejoins the recorded stream), and
+    with the workspace cap so small that each lane runs several chunks.  The automatic choice takes two
+    lanes for the GPT-2-small list and one for the conv list and for a handful of matrices."""
+    from muon_amd import plan
+    shapes = [(768, 2304), (768, 768), (3072, 768), (1024, 1536), (256, 576), (128, 8192), (64, 24, 3, 3),
+              (512, 2304), (1280, 1024), (3, 200, 136)]
+    torch.manual_seed(1500)
+    init = [torch.randn(*s) * 0.02 for s in shapes]
+    grads = [[torch.randn(*s) * 1e-3 for s in shapes] for _ in range(3)]
+    adam_init = torch.randn(50, 8) * 0.02
+
+    def run(lanes, **kw):
+        saved, plan.LANES = plan.LANES, lanes
+        try:
+            pm = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+            pa = [torch.nn.Parameter(adam_init.clone().cuda())]
+            opt = M.SingleDeviceMuonWithAuxAdam([
+                dict(params=pm, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01),
+                dict(params=pa, use_muon=False, lr=3e-4, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)], **kw)
+            for gs in grads:
+                for p, g in zip(pm, gs):
+                    p.grad = g.clone().cuda()
+                pa[0].grad = torch.ones_like(pa[0]) * 1e-3
+                opt.step()
+                torch.cuda.synchronize()          # eager work and a synchronisation between replays
+            (eng,) = opt._muon_engines.values()
+            return [p.detach().cpu() for p in pm + pa], eng
+        finally:
+            plan.LANES = saved
+
+    one, eng1 = run("1")
+    assert len(eng1.lane_runtimes) == 1
+    for kw in ({}, {"use_graph": True}, {"workspace_bytes": 24 << 20}):
+        two, eng2 = run("2", **kw)
+        assert len(eng2.lane_runtimes) == 2 and eng2.lane_streams[1] is not None
+        if "workspace_bytes" in kw:
+            assert all(len(lane) > 1 for lane in eng2.lane_runtimes)
+        assert sorted(l.index for rt in eng2.runtimes for l in rt.chunk.layouts) == list(range(len(eng2.shapes)))
+        for a, b in zip(one, two):
+            assert torch.equal(a, b), kw
+    gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    conv = [(64, 216), (256, 576), (256, 2304), (256, 2304), (512, 2304), (512, 4608), (512, 4608), (512, 4608),
+            (128, 16384), (16384, 128)]
+    assert len(plan.plan_lanes(gpt2, 5, True, 16 << 30)) == 2
+    assert len(plan.plan_lanes(conv, 5, True, 16 << 30)) == 1
+    assert len(plan.plan_lanes(gpt2[:4], 5, True, 16 << 30)) == 1
+    assert len(plan.plan_lanes(gpt2, 5, True, 16 << 30, allow_lanes=False)) == 1
