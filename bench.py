@@ -32,7 +32,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM-side bytes per ns_gemm launch: NOT measured by this script.  The figure comes from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE, scaled by what the counters read for
 # a 1 GiB copy, averaged over the launches of a step); the summary file is named beside it.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": (2.96e10, "profiles/hbm_traffic_llama3-8b_step.md")}
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = {"llama3-8b": (3.02e10, "profiles/hbm_traffic_llama3-8b_step.md")}
 
 TOL_NS_BF16, TOL_NS_FP32, TOL_PARAM, TOL_ADAM = 2e-2, 3e-2, 1e-3, 1e-5
 
