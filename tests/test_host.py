@@ -602,3 +602,28 @@ def test_update_launches_of_matrices_with_ragged_super_blocks_deal_whole_matrice
     finally:
         plan.WHOLE_MATRIX_GROUPS = old
     assert (c2.full_jobs == ref).all()
+
+
+def test_lanes_split_mid_sized_groups_and_nothing_else():
+    """Two lanes (every other matrix of the sorted list, planned separately) for a group that is one
+    chunk of at least 8 matrices with launches of 60 us to 1 ms; one lane for short launches (conv),
+    long ones (Llama, a batch of 4096 x 4096), a handful of matrices, several chunks, and on request."""
+    gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
+    lanes = plan.plan_lanes(gpt2, 5, True, 16 << 30)
+    assert len(lanes) == 2 and all(len(lane) == 1 and lane[0].nmat == 24 for lane in lanes)
+    idx = [sorted(lay.index for c in lane for lay in c.layouts) for lane in lanes]
+    assert sorted(idx[0] + idx[1]) == list(range(48)) and not set(idx[0]) & set(idx[1])
+    for lane in lanes:       # the same mix of shapes in both
+        assert sorted((lay.m, lay.n) for lay in lane[0].layouts) == sorted([(768, 2304), (768, 768), (768, 3072), (768, 3072)] * 6)
+        assert lane[0].update_class == 1
+    conv = [(64, 216), (256, 576), (256, 2304), (256, 2304), (512, 2304), (512, 4608), (512, 4608), (512, 4608),
+            (128, 16384), (16384, 128)]
+    llama = [(4096, 4096)] * 64 + [(1024, 4096)] * 64 + [(14336, 4096)] * 64 + [(4096, 14336)] * 32
+    for shapes in (conv, llama, [(4096, 4096)] * 32, gpt2[:4]):
+        assert len(plan.plan_lanes(shapes, 5, True, 16 << 30)) == 1
+    assert len(plan.plan_lanes(gpt2, 5, True, 16 << 30, allow_lanes=False)) == 1
+    assert len(plan.plan_lanes(gpt2, 5, True, 64 << 20)) == 1                     # several chunks: one lane
+    # a group whose halves would fall back to the small update tiles stays whole
+    few = [(768, 3072)] * 8
+    (c,) = plan.plan_chunks(few, 5, True, 16 << 30)
+    assert c.update_class == 1 and len(plan.plan_lanes(few, 5, True, 16 << 30)) == 1
