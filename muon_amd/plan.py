@@ -489,8 +489,7 @@ def _shape_order_key(shapes, i):
 
 
 LANES = os.environ.get("MUON_AMD_LANES", "auto")        # "auto", or a number of lanes to force ("1" switches them off)
-LANE_MIN_MATRICES = 8
-LANE_LAUNCH_US = (60.0, 1000.0)
+LANE_UPDATE_TILES = (600, 2600)
 
 
 def plan_lanes(shapes, steps: int, reference_rounding: bool, workspace_cap: int, variant: str = "ns5",
@@ -498,22 +497,27 @@ def plan_lanes(shapes, steps: int, reference_rounding: bool, workspace_cap: int,
     """-> lanes, each a list of chunks.  Lanes have workspaces of their own and run side by side on
     streams of their own, so that the launches of one fill the CUs that the last, partly filled
     rounds of the other's leave idle (every launch is persistent: while one runs in full, the other
-    lane's next launch waits for CUs and starts where they free up).  Two lanes, each with every
-    other matrix of the sorted list, when the matrices make one chunk of at least 8 whose launches
-    are estimated at 60 us to 1 ms each: measured on the Muon part of a step, GPT-2-124M 2.07 ->
-    1.975 ms, 96 matrices of m = 512 1.60 -> 1.52, 96 of m = 1024 7.68 -> 7.51, 48 of m = 1280 7.10 ->
-    6.87 ms.  Not for short launches (the conv configuration: 0.43 -> 0.45 ms, and the host then
-    issues two streams' worth of them) nor for long ones (the Llama-3-8B matrices: 438 -> 448 ms; three
-    and four lanes were no better than two anywhere).  Which lane computes a matrix does not change
-    its bits."""
+    lane's next launch waits for CUs and starts where they free up).
+
+    Two lanes, each with every other matrix of the sorted list, are taken for what measured faster
+    that way: one chunk of the 128 x 128 class whose update products run in 600 to 2600 tiles of
+    256 x 256, a few rounds with a ragged last one (Muon part of a step: the 48 GPT-2-124M matrices
+    2.07 -> 1.975 ms, 96 matrices of m = 512 1.60 -> 1.52, 96 of GPT-2's shapes 4.01 -> 3.94, 24 of them
+    1.08 -> 1.08).  Everything else measured slower in two lanes and stays in one: more tiles (192
+    GPT-2 shapes 7.81 -> 8.2 ms), chunks whose update products stay in 128 x 128 tiles (m = 896, 640,
+    384: +4 to +20 %), the 256 x 256 class (m = 1024 and 1280 gain 2-3 % with 96 / 48 matrices and lose
+    7-8 % with twice as many; m = 1536, 2048, 4096 and the Llama-3-8B matrices lose 2-14 %: two large
+    kernels side by side evict each other's panels), and short launches (conv: the host then issues
+    two streams' worth of them).  Three lanes measured like two, four slower.  Which lane computes a
+    matrix does not change its bits."""
     chunks = plan_chunks(shapes, steps, reference_rounding, workspace_cap, variant)
     n = 1
     if allow_lanes and LANES != "auto":
         n = max(1, min(int(LANES), len(shapes)))
-    elif allow_lanes and len(chunks) == 1 and chunks[0].nmat >= LANE_MIN_MATRICES:
+    elif allow_lanes and len(chunks) == 1:
         c = chunks[0]
-        est, _ = _chunk_time_us([(lay.rows, lay.cols) for lay in c.layouts], c.tile_class)
-        if LANE_LAUNCH_US[0] <= est / 3 <= LANE_LAUNCH_US[1]:
+        if (c.tile_class == 0 and c.update_class == 1 and
+                LANE_UPDATE_TILES[0] <= len(c.full_jobs) <= LANE_UPDATE_TILES[1]):
             n = 2
     if n == 1:
         return [chunks]

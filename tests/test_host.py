@@ -604,10 +604,11 @@ def test_update_launches_of_matrices_with_ragged_super_blocks_deal_whole_matrice
     assert (c2.full_jobs == ref).all()
 
 
-def test_lanes_split_mid_sized_groups_and_nothing_else():
-    """Two lanes (every other matrix of the sorted list, planned separately) for a group that is one
-    chunk of at least 8 matrices with launches of 60 us to 1 ms; one lane for short launches (conv),
-    long ones (Llama, a batch of 4096 x 4096), a handful of matrices, several chunks, and on request."""
+def test_lanes_split_groups_like_gpt2_small_and_nothing_else():
+    """Two lanes (every other matrix of the sorted list, planned separately) for one chunk of the
+    128 x 128 class whose update products run in 600-2600 tiles of 256 x 256; one lane for everything
+    that measured slower in two: more tiles, update products in small tiles, the 256 x 256 class, short
+    launches, several chunks, and on request."""
     gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
     lanes = plan.plan_lanes(gpt2, 5, True, 16 << 30)
     assert len(lanes) == 2 and all(len(lane) == 1 and lane[0].nmat == 24 for lane in lanes)
@@ -616,14 +617,16 @@ def test_lanes_split_mid_sized_groups_and_nothing_else():
     for lane in lanes:       # the same mix of shapes in both
         assert sorted((lay.m, lay.n) for lay in lane[0].layouts) == sorted([(768, 2304), (768, 768), (768, 3072), (768, 3072)] * 6)
         assert lane[0].update_class == 1
+    assert len(plan.plan_lanes([(512, 1536), (512, 512), (512, 2048), (2048, 512)] * 24, 5, True, 16 << 30)) == 2
+    assert len(plan.plan_lanes(gpt2 * 2, 5, True, 16 << 30)) == 2
     conv = [(64, 216), (256, 576), (256, 2304), (256, 2304), (512, 2304), (512, 4608), (512, 4608), (512, 4608),
             (128, 16384), (16384, 128)]
     llama = [(4096, 4096)] * 64 + [(1024, 4096)] * 64 + [(14336, 4096)] * 64 + [(4096, 14336)] * 32
-    for shapes in (conv, llama, [(4096, 4096)] * 32, gpt2[:4]):
+    one = (conv, llama, [(4096, 4096)] * 32, gpt2[:4], gpt2 * 4,
+           [(896, 2688), (896, 896), (896, 3584), (3584, 896)] * 12,            # update products in 128 x 128 tiles
+           [(1024, 3072), (1024, 1024), (1024, 4096), (4096, 1024)] * 24,       # the 256 x 256 class
+           [(1536, 4608), (1536, 1536), (1536, 6144), (6144, 1536)] * 8)
+    for shapes in one:
         assert len(plan.plan_lanes(shapes, 5, True, 16 << 30)) == 1
     assert len(plan.plan_lanes(gpt2, 5, True, 16 << 30, allow_lanes=False)) == 1
     assert len(plan.plan_lanes(gpt2, 5, True, 64 << 20)) == 1                     # several chunks: one lane
-    # a group whose halves would fall back to the small update tiles stays whole
-    few = [(768, 3072)] * 8
-    (c,) = plan.plan_chunks(few, 5, True, 16 << 30)
-    assert c.update_class == 1 and len(plan.plan_lanes(few, 5, True, 16 << 30)) == 1
