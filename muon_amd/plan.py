@@ -264,12 +264,16 @@ def whole_matrix_group(tiles_per_matrix, default: int) -> int:
     """Group size for a launch of 256 x 256 tiles over matrices whose tile rows do not fill the
     super-block (3 or 5 tile rows against its 4): groups of `default` jobs then straddle super-blocks
     and matrices, and several XCDs fetch the same small B and X.  Whole matrices per XCD instead: the
-    least common multiple of the matrices' tile counts when that is at most eight super-blocks, else
-    the largest count (measured on the update launches of GPT-2-124M, m = 768: 0.187 -> 0.180 ms, and
-    of m = 1280: 0.647 -> 0.622 ms; matrices with 4 or 16 tile rows are best left in super-blocks)."""
+    least common multiple of the matrices' tile counts, or else the largest count, when that is at
+    most four super-blocks (measured on the update launches of GPT-2-124M, m = 768, groups of 108: 0.187
+    -> 0.180 ms, and of m = 1280, groups of 100: 0.647 -> 0.622 ms).  Larger matrices keep the
+    super-block groups: m = 1536 and 1792 (groups of 144, 147) measured the same either way, m = 2304
+    (324) 2 % slower in whole matrices; matrices with 4 or 16 tile rows are best left in super-blocks."""
     counts = sorted(set(int(t) for t in tiles_per_matrix))
-    g = int(np.lcm.reduce(counts))
-    return g if g <= 8 * default else max(counts)
+    for g in (int(np.lcm.reduce(counts)), max(counts)):
+        if g <= 4 * default:
+            return g
+    return default
 
 
 class ChunkPlan:

@@ -584,7 +584,8 @@ def test_update_launches_of_matrices_with_ragged_super_blocks_deal_whole_matrice
     in groups of 108 jobs = 4, 12 or 3 whole matrices, so an XCD sees few matrices; matrices whose
     tile rows fill the super-blocks (m = 1024, 4096) keep the super-block groups."""
     assert plan.whole_matrix_group([27, 9, 36, 36], 32) == 108
-    assert plan.whole_matrix_group([75, 25, 100], 32) == 100           # lcm 300 is more than eight super-blocks
+    assert plan.whole_matrix_group([75, 25, 100], 32) == 100           # lcm 300 is more than four super-blocks
+    assert plan.whole_matrix_group([243, 81, 324], 32) == 32           # matrices this large keep the super-block groups
     gpt2 = [(768, 2304), (768, 768), (768, 3072), (3072, 768)] * 12
     (c,) = plan.plan_chunks(gpt2, 5, True, 16 << 30)
     assert c.update_class == 1 and len(c.full_jobs) == 1296
