@@ -371,10 +371,12 @@ class MuonGroupEngine:
         h = self._hyper
         return (id(self), h["nesterov"], h["mutate_grad"], h["eps"], self._skip)
 
-    def enqueue(self, scalars_ptr: int = 0):
+    def enqueue(self, scalars_ptr: int = 0, join: bool = True):
         """The launches of every lane: the first lane on the current stream, the others on their own
         streams, which wait for what the current stream holds so far (the descriptor uploads of
-        `prepare`, the gradients) and which the current stream waits for before it goes on."""
+        `prepare`, the gradients) and which the current stream waits for before it goes on -- here,
+        or (join=False) when the caller calls `join`, having enqueued work that does not depend on
+        these matrices in between (the Adam launch of the same step)."""
         h = self._hyper
         main = torch.cuda.current_stream(self.device)
         for side in self.lane_streams[1:]:
@@ -385,6 +387,12 @@ class MuonGroupEngine:
                     rt.run(h["one_minus_beta"], h["beta"], h["nesterov"], h["mutate_grad"], h["eps"], h["lr"],
                            h["wd_factor"], scalars_ptr=scalars_ptr,
                            momentum_done=self._skip if (li == 0 and n == 0) else frozenset())
+        if join:
+            self.join()
+
+    def join(self):
+        """The current stream waits for the lanes that run on streams of their own."""
+        main = torch.cuda.current_stream(self.device)
         for side in self.lane_streams[1:]:
             main.wait_stream(side)
 
@@ -495,7 +503,10 @@ class AdamGroupEngine:
     def structure_key(self):
         return (id(self),)
 
-    def enqueue(self, scalars_ptr: int = 0):
+    def join(self):
+        pass
+
+    def enqueue(self, scalars_ptr: int = 0, join: bool = True):
         lib = _lib.load()
         lr, wd_factor, w1, w2, eps, bias1, bias2 = self._hyper
         _launch("adam", self.nbytes, lambda: _lib.check(lib.muon_amd_adam(
@@ -540,7 +551,9 @@ class StepGraph:
             base = self.scalars.data_ptr()
             with torch.cuda.graph(graph):
                 for e, off in zip(engines, offsets):
-                    e.enqueue(base + 4 * off)
+                    e.enqueue(base + 4 * off, join=False)
+                for e in engines:
+                    e.join()
             self.graph, self.key = graph, key
         self.graph.replay()
         self.replays += 1

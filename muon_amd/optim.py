@@ -326,8 +326,12 @@ class _MuonBase(torch.optim.Optimizer):
                             graph = self._graphs[device] = StepGraph(device)
                         graph.run(engines)
                     else:
+                        # lanes on streams of their own are joined after everything is enqueued: the
+                        # Adam launch does not wait for the last Muon launch of another lane
                         for eng in engines:
-                            eng.enqueue()
+                            eng.enqueue(join=False)
+                        for eng in engines:
+                            eng.join()
             for dst, src in self._writebacks:
                 dst.copy_(src)
         finally:
