@@ -550,10 +550,12 @@ class StepGraph:
             graph = torch.cuda.CUDAGraph()
             base = self.scalars.data_ptr()
             with torch.cuda.graph(graph):
-                for e, off in zip(engines, offsets):
-                    e.enqueue(base + 4 * off, join=False)
-                for e in engines:
-                    e.join()
+                try:
+                    for e, off in zip(engines, offsets):
+                        e.enqueue(base + 4 * off, join=False)
+                finally:
+                    for e in engines:
+                        e.join()
             self.graph, self.key = graph, key
         self.graph.replay()
         self.replays += 1

@@ -328,10 +328,12 @@ class _MuonBase(torch.optim.Optimizer):
                     else:
                         # lanes on streams of their own are joined after everything is enqueued: the
                         # Adam launch does not wait for the last Muon launch of another lane
-                        for eng in engines:
-                            eng.enqueue(join=False)
-                        for eng in engines:
-                            eng.join()
+                        try:
+                            for eng in engines:
+                                eng.enqueue(join=False)
+                        finally:                  # also when a launch was refused: nothing stays unjoined
+                            for eng in engines:
+                                eng.join()
             for dst, src in self._writebacks:
                 dst.copy_(src)
         finally:
